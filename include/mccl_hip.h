@@ -1,0 +1,207 @@
+/*
+ * mccl_hip.h -- C ABI of the MI355X (gfx950) implementation of MCCL's per-rank
+ * data-parallel compute path: chunk fold, AVG scale, ring-order W-way fold,
+ * top-k compression with error feedback, decompress and rank-ordered sparse
+ * accumulate.
+ *
+ * Conventions
+ *   - Every pointer is DEVICE memory unless its name starts with `host_`.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *     Calls only enqueue work; completion is observed through the stream, a
+ *     fence ticket (below) or mccl_hip_sync().
+ *   - Return value: MCCL_HIP_OK or a negative MCCL_HIP_ERR_* code.  Nothing
+ *     throws, nothing takes ownership of caller memory.
+ *   - `dtype` uses the numeric values of at::ScalarType, `op` those of
+ *     c10d::ReduceOp::RedOpType, so a torch binding can pass them through.
+ *
+ * Each entry point names the reference interface it replaces (paths are
+ * relative to the reference checkout).
+ */
+#ifndef MCCL_HIP_H
+#define MCCL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MCCL_HIP_ABI_VERSION 1
+
+/* ---- status codes ------------------------------------------------------ */
+#define MCCL_HIP_OK 0
+#define MCCL_HIP_ERR_OP (-1)        /* "Unsupported ReduceOp" (csrc/metal/MetalKernels.mm:798-800) */
+#define MCCL_HIP_ERR_DTYPE (-2)     /* no kernel for this element type (MetalKernels.mm:542-544)   */
+#define MCCL_HIP_ERR_CAPACITY (-3)  /* "TopK compress: buffer too small" (TopKCompression.cpp:94)  */
+#define MCCL_HIP_ERR_SIZE (-4)      /* "TopK decompress: size mismatch" (TopKCompression.cpp:138)  */
+#define MCCL_HIP_ERR_INDEX (-5)     /* "TopK decompress: index out of bounds" (:148)               */
+#define MCCL_HIP_ERR_ARG (-6)       /* null pointer, zero/oversized count, bad ratio, bad world size */
+#define MCCL_HIP_ERR_RUNTIME (-7)   /* a HIP runtime call failed; see mccl_hip_last_hip_error()     */
+#define MCCL_HIP_ERR_WORKSPACE (-8) /* workspace smaller than mccl_hip_topk_workspace_bytes()       */
+#define MCCL_HIP_ERR_TIMEOUT (-9)   /* fence wait exceeded its limit (csrc/metal/EventSync.mm:37-71) */
+
+/* ---- element types (at::ScalarType values) ------------------------------ */
+#define MCCL_HIP_U8 0
+#define MCCL_HIP_I32 3
+#define MCCL_HIP_I64 4
+#define MCCL_HIP_F16 5
+#define MCCL_HIP_F32 6
+#define MCCL_HIP_BOOL 11
+#define MCCL_HIP_BF16 15
+
+/* ---- reduce ops (c10d::ReduceOp::RedOpType values) ---------------------- */
+#define MCCL_HIP_SUM 0
+#define MCCL_HIP_AVG 1 /* folds like SUM; the caller scales afterwards */
+#define MCCL_HIP_PRODUCT 2
+#define MCCL_HIP_MIN 3
+#define MCCL_HIP_MAX 4
+
+/* ---- ring schedules ----------------------------------------------------- */
+#define MCCL_HIP_RING_BASIC 0   /* ws chunks of ceil(n/ws)       (ProcessGroupMCCL.cpp:1989-2034) */
+#define MCCL_HIP_RING_CHUNKED 1 /* 2*ws chunks of ceil(n/(2*ws)) (ProcessGroupMCCL.cpp:1725-1772) */
+
+#define MCCL_HIP_MAX_WORLD 64
+
+/* Largest element count a single call accepts (the reference caps kernels at
+ * UINT32_MAX elements, csrc/metal/MetalKernels.mm:292-299; this library takes
+ * 64-bit counts up to 2^40). */
+#define MCCL_HIP_MAX_ELEMS (1ull << 40)
+
+/* ---- library state ------------------------------------------------------ */
+
+/* Replaces metal_kernels_init() (csrc/metal/MetalKernels.mm:360-366) and
+ * event_sync_init() (csrc/metal/EventSync.mm:76-100).  Idempotent and
+ * thread-safe.  Fails with MCCL_HIP_ERR_RUNTIME when no gfx950 device is
+ * current. */
+int mccl_hip_init(void);
+int mccl_hip_abi_version(void);
+const char* mccl_hip_strerror(int code);
+/* hipError_t value of the most recent failing runtime call on this thread. */
+int mccl_hip_last_hip_error(void);
+
+/* ---- binary folds: one ring step ---------------------------------------- */
+
+/* dst[i] = dst[i] (op) src[i], in place on dst, dst = local chunk, src =
+ * incoming chunk.  Replaces metal_reduce_op / metal_accumulate_chunk /
+ * metal_elementwise_{min,max,product} (csrc/metal/MetalKernels.hpp:17-31,
+ * MetalKernels.mm:521-565,:712-802) and cpu_reduce_op[_half|_bf16|_integral]
+ * (csrc/metal/AccelerateOps.hpp:21-59).  F16/BF16: widen, one fp32 operation,
+ * one round-to-nearest-even narrow.  MIN/MAX are compare-selects
+ * `(src < dst) ? src : dst`.  dst and src need only element alignment. */
+int mccl_hip_fold2(void* dst, const void* src, uint64_t n, int dtype, int op, void* stream);
+
+/* buf[i] = buf[i] * scale (one fp32 multiply; F16/BF16 multiply in fp32 and
+ * round once).  Integral types: T(float(x) * scale), truncating for
+ * I64/U8/BOOL and rounding half away from zero for I32.  Replaces
+ * metal_scale_inplace (MetalKernels.mm:568-613, csrc/metal/shaders.metal:
+ * 233-332,:622-665) and cpu_scale_inplace* (AccelerateOps.mm:103-120). */
+int mccl_hip_scale(void* buf, uint64_t n, int dtype, float scale, void* stream);
+
+/* dst[i] = (dst[i] + src[i]) * scale with the sum rounded to fp32 before the
+ * multiply.  Integral types run the add and then the scale rule above.
+ * Replaces metal_accumulate_and_scale (MetalKernels.mm:616-675) and
+ * cpu_accumulate_and_scale* (AccelerateOps.mm:122-142). */
+int mccl_hip_fold2_scale(void* dst, const void* src, uint64_t n, int dtype, float scale,
+                         void* stream);
+
+/* ---- W-way fold in ring-step order -------------------------------------- */
+
+/* The reduce half of a ring allreduce over `ws` simulated ranks whose buffers
+ * all live in this GPU's memory.  host_in[r] is rank r's buffer of n_total
+ * elements; out receives the reduced result (out may alias one host_in[r]).
+ * The n_total elements are cut into buckets of bucket_elems (the last one may
+ * be shorter; bucket_elems >= n_total means one bucket), every bucket into the
+ * schedule's chunks, and chunk c is folded left to right starting at the rank
+ * that owns it in the reference's step plan
+ * (send_idx/recv_idx, ProcessGroupMCCL.cpp:1754-1762,:2016-2024; receive side
+ * reduces local (op)= incoming, :492-512):
+ *     acc = x[s]; for j = 1..ws-1: acc = x[(s+j) % ws] (op) acc
+ * then, if apply_scale, one multiply by `scale` (the AVG tail,
+ * ProcessGroupMCCL.cpp:1954-1956,:2177-2179).
+ * F16/BF16: stepwise != 0 rounds the partial to the element type after every
+ * step (what the reference sends between ranks); stepwise == 0 keeps the
+ * partial in fp32 and rounds once at the end. */
+int mccl_hip_ring_fold(void* out, const void* const* host_in, int ws, uint64_t n_total,
+                       uint64_t bucket_elems, int schedule, int dtype, int op, int apply_scale,
+                       float scale, int stepwise, void* stream);
+
+/* ---- top-k compression with error feedback ------------------------------ */
+
+/* k = max(1, uint32(count * ratio)), product in double
+ * (csrc/compression/TopKCompression.cpp:45-47). */
+uint32_t mccl_hip_topk_k(uint64_t count, double ratio);
+/* TopKCompressor::max_compressed_size (TopKCompression.cpp:154-158). */
+uint64_t mccl_hip_topk_max_compressed_size(uint64_t nbytes, double ratio);
+/* Bytes of scratch mccl_hip_topk_compress needs for this shape. */
+uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems);
+
+/* TopKCompressor::compress (TopKCompression.cpp:38-120) for every bucket of a
+ * gradient in one call.  grad and residual hold n_total fp32 elements, cut
+ * into buckets of bucket_elems (last may be shorter; bucket_elems >= n_total
+ * means one bucket = one reference compress() call).  Per bucket b of count
+ * n_b: residual += grad; the k_b = mccl_hip_topk_k(n_b, ratio) elements of
+ * largest magnitude are written in ascending index order (indices relative to
+ * the bucket) as [u32 k_b][k_b x {u32 index, f32 value}] at
+ * wire + b * wire_stride, and residual is zeroed at those elements.  Ties at
+ * the threshold magnitude go to the lower index.  wire_stride must be a
+ * multiple of 4 and at least 4 + 8 * k_b for the largest bucket
+ * (else MCCL_HIP_ERR_CAPACITY).  NaN input is outside the contract. */
+int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
+                           uint64_t bucket_elems, double ratio, void* wire,
+                           uint64_t wire_stride, void* workspace, uint64_t workspace_bytes,
+                           void* stream);
+
+/* TopKCompressor::decompress (TopKCompression.cpp:122-152): dense[0..count) is
+ * zeroed, then dense[index] = value for every pair.  wire_bytes is the size
+ * that arrived with the payload; it must equal 4 + 8 * k for the k stored in
+ * the payload.  Violations are reported through *status (a device int the
+ * caller zeroes beforehand and reads after the stream has drained): it
+ * receives MCCL_HIP_ERR_SIZE or MCCL_HIP_ERR_INDEX; offending pairs are
+ * skipped.  status may be NULL. */
+int mccl_hip_topk_decompress(const void* wire, uint64_t wire_bytes, float* dense, uint64_t count,
+                             int* status, void* stream);
+
+/* Decompress + accumulate of `ws` ranks' payloads into one dense buffer, the
+ * sparse equivalent of decompressing every peer's payload and folding the
+ * dense buffers in ascending rank order, then the AVG multiply
+ * (ProcessGroupMCCL.cpp:1692-1709,:2272-2296):
+ *     acc = +0.0; for r = 0..ws-1: acc[idx] += val for r's pairs; acc *= scale
+ * host_wires[r] is rank r's payload buffer laid out like the output of
+ * mccl_hip_topk_compress (bucket b at + b * wire_stride, indices relative to
+ * the bucket).  Every element of acc is written exactly once.  Each payload's
+ * k is read on the device; 4 + 8k > wire_stride or an index outside its bucket
+ * sets *status (as above) and the offending pairs are skipped.  Pairs within
+ * one payload must have ascending indices (what compress emits). */
+int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems,
+                               const void* const* host_wires, int ws, uint64_t wire_stride,
+                               int apply_scale, float scale, int* status, void* stream);
+
+/* ---- ordering ----------------------------------------------------------- */
+
+/* Replaces next_fence_event_value() + signal_mccl_fence_gpu()
+ * (csrc/metal/EventSync.mm:189-200): records an event on `stream` and returns
+ * its ticket (monotonic, never 0) in *ticket. */
+int mccl_hip_fence_signal(void* stream, uint64_t* ticket);
+/* Replaces wait_for_mccl_fence() (EventSync.mm:202-206): blocks the host until
+ * everything enqueued before the ticket has completed.  timeout_ms <= 0 uses
+ * the reference's 30 s limit.  Tickets older than the event ring are complete
+ * by construction. */
+int mccl_hip_fence_wait(uint64_t ticket, int timeout_ms);
+/* Non-blocking: 1 complete, 0 pending, negative on error. */
+int mccl_hip_fence_query(uint64_t ticket);
+/* Makes `stream` wait (on the device) for the ticket; the analogue of
+ * block_mps_on_mccl() (EventSync.mm:173-187). */
+int mccl_hip_fence_block_stream(uint64_t ticket, void* stream);
+/* Replaces metal_sync() / metal_sync_queue_only() (MetalKernels.mm:816-824). */
+int mccl_hip_sync(void* stream);
+
+/* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
+/* keys: "fold_blocks_per_cu", "fold_unroll", "nontemporal", "topk_path"  */
+int mccl_hip_set_tuning(const char* key, int value);
+int mccl_hip_get_tuning(const char* key);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MCCL_HIP_H */

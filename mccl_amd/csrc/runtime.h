@@ -1,0 +1,54 @@
+// Host-side state shared by the kernel launchers: device properties, tuning
+// knobs, HIP error capture.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mccl_hip.h"
+
+namespace mcclhip {
+
+struct DeviceInfo {
+    int device = -1;
+    int num_cus = 256;
+    bool ok = false;
+};
+
+// Lazily initialised properties of the current device (mccl_hip_init).
+const DeviceInfo& device_info();
+
+struct Tuning {
+    int fold_blocks_per_cu = 8;  // resident 256-thread blocks per CU for streaming kernels
+    int fold_unroll = 4;         // 16-byte vectors in flight per thread and operand (1, 2 or 4)
+    int nontemporal = 0;         // 1: streaming loads/stores carry the `nt` hint
+    int topk_path = 0;           // 0 auto, 1 force the multi-pass exact path
+};
+Tuning& tuning();
+
+void record_hip_error(hipError_t e);
+
+#define MCCLHIP_TRY(expr)                            \
+    do {                                             \
+        hipError_t _e = (expr);                      \
+        if (_e != hipSuccess) {                      \
+            ::mcclhip::record_hip_error(_e);         \
+            return MCCL_HIP_ERR_RUNTIME;             \
+        }                                            \
+    } while (0)
+
+// Call after every kernel launch: launch-time errors surface here.
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        record_hip_error(e);
+        return MCCL_HIP_ERR_RUNTIME;
+    }
+    return MCCL_HIP_OK;
+}
+
+inline uint32_t clamp_u32(uint64_t v, uint64_t lo, uint64_t hi) {
+    return (uint32_t)(v < lo ? lo : (v > hi ? hi : v));
+}
+
+}  // namespace mcclhip

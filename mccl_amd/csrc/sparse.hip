@@ -1,0 +1,185 @@
+// Decompress and rank-ordered sparse accumulate of top-k payloads for gfx950.
+//
+// Payload layout (csrc/compression/TopKCompression.cpp:93-113):
+//   [u32 k][k x {u32 index, f32 value}], little endian, indices ascending.
+//
+// decompress: dense = 0, dense[index] = value (TopKCompression.cpp:122-152).
+//
+// sparse accumulate: the reference decompresses every peer's payload into a
+// dense buffer and folds the dense buffers in ascending rank order
+// (csrc/backend/ProcessGroupMCCL.cpp:1692-1709,:2272-2296).  Here each block
+// owns one 4096-element tile of the output, keeps it in LDS starting at +0.0,
+// and for rank 0, 1, ... adds that rank's pairs that fall inside the tile
+// (found by binary search in the sorted payload; indices are unique within a
+// rank, so a rank's adds never collide), then writes the tile once, scaled.
+// HBM traffic is the algorithmic minimum: every payload read once, every output
+// element written once.
+#include "common.hip.h"
+#include "runtime.h"
+
+namespace mcclhip {
+
+namespace {
+
+constexpr int kAccTile = 4096;
+
+__global__ __launch_bounds__(kBlock) void k_fill_zero(float* p, uint64_t n) {
+    // 16-byte stores over the aligned body, scalars at both ends
+    uint64_t head = ((16 - ((uintptr_t)p & 15)) & 15) / 4;
+    if (head > n) head = n;
+    const uint64_t nvec = (n - head) / 4;
+    u4a* v = (u4a*)(p + head);
+    const u4a z = {0u, 0u, 0u, 0u};
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (uint64_t)gridDim.x * kBlock)
+        v[i] = z;
+    const uint64_t g = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g < head) p[g] = 0.0f;
+    const uint64_t tail = head + nvec * 4;
+    if (g < 4 && tail + g < n) p[tail + g] = 0.0f;
+}
+
+__global__ __launch_bounds__(kBlock) void k_scatter(const uint32_t* wire, uint32_t expected_k, float* dense,
+                                                    uint64_t count, int* status) {
+    const uint32_t k = wire[0];
+    if (k != expected_k) {
+        if (status && blockIdx.x == 0 && threadIdx.x == 0) *status = MCCL_HIP_ERR_SIZE;
+        return;
+    }
+    for (uint64_t p = (uint64_t)blockIdx.x * kBlock + threadIdx.x; p < k; p += (uint64_t)gridDim.x * kBlock) {
+        const uint32_t idx = wire[1 + 2 * p];
+        const uint32_t val = wire[2 + 2 * p];
+        if (idx < count) dense[idx] = u2f(val);
+        else if (status) *status = MCCL_HIP_ERR_INDEX;
+    }
+}
+
+struct WirePtrs {
+    const uint8_t* w[MCCL_HIP_MAX_WORLD];
+};
+
+// First pair position in [0, k) whose index is >= target (k if none).
+__device__ __forceinline__ uint32_t lower_bound_idx(const uint32_t* pairs, uint32_t k, uint32_t target) {
+    uint32_t lo = 0, hi = k;
+    while (lo < hi) {
+        const uint32_t mid = lo + ((hi - lo) >> 1);
+        if (pairs[2 * (uint64_t)mid] < target) lo = mid + 1;
+        else hi = mid;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(kBlock) void k_sparse_accumulate(float* acc, uint64_t n_total,
+                                                              uint64_t bucket_elems, WirePtrs wires, int ws,
+                                                              uint64_t wire_stride, int apply_scale,
+                                                              float scale, int* status) {
+    __shared__ float tile[kAccTile];
+    __shared__ uint32_t lo_s[MCCL_HIP_MAX_WORLD], hi_s[MCCL_HIP_MAX_WORLD];
+    const uint32_t b = blockIdx.y, t = blockIdx.x;
+    const uint64_t bstart = (uint64_t)b * bucket_elems;
+    const uint64_t bn = (n_total - bstart) < bucket_elems ? (n_total - bstart) : bucket_elems;
+    const uint64_t tstart = (uint64_t)t * kAccTile;
+    if (tstart >= bn) return;
+    const uint32_t tlen = (uint32_t)((bn - tstart) < kAccTile ? (bn - tstart) : kAccTile);
+    const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
+
+    for (int i = threadIdx.x; i < kAccTile; i += kBlock) tile[i] = 0.0f;
+    // range of every rank's pairs inside this tile: thread r -> lower end, thread ws + r -> upper end
+    if (threadIdx.x < 2 * ws) {
+        const int r = threadIdx.x < ws ? threadIdx.x : threadIdx.x - ws;
+        const uint32_t* wp = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride);
+        uint32_t k = wp[0];
+        if (k > kmax) {
+            if (status) *status = MCCL_HIP_ERR_SIZE;
+            k = 0;
+        }
+        if (threadIdx.x < ws) {
+            lo_s[r] = lower_bound_idx(wp + 1, k, (uint32_t)tstart);
+        } else {
+            hi_s[r] = lower_bound_idx(wp + 1, k, (uint32_t)(tstart + tlen));
+            // the block that owns the bucket's last tile also checks the largest index
+            if (tstart + tlen == bn && k > 0 && wp[1 + 2 * (uint64_t)(k - 1)] >= bn && status)
+                *status = MCCL_HIP_ERR_INDEX;
+        }
+    }
+    __syncthreads();
+    for (int r = 0; r < ws; r++) {
+        const uint32_t* pairs = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride) + 1;
+        const uint32_t lo = lo_s[r], hi = hi_s[r];
+        for (uint32_t p = lo + threadIdx.x; p < hi; p += kBlock) {
+            const uint32_t off = pairs[2 * (uint64_t)p] - (uint32_t)tstart;
+            const float v = u2f(pairs[2 * (uint64_t)p + 1]);
+            if (off < tlen) tile[off] = tile[off] + v;
+            else if (status) *status = MCCL_HIP_ERR_INDEX;  // unsorted payload
+        }
+        __syncthreads();
+    }
+    float* out = acc + bstart + tstart;
+    if (tlen == kAccTile && (((uintptr_t)out & 15) == 0)) {
+        for (int i = threadIdx.x; i < kAccTile / 4; i += kBlock) {
+            u4a v;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float x = tile[4 * i + q];
+                v[q] = f2u(apply_scale ? x * scale : x);
+            }
+            ((u4a*)out)[i] = v;
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < tlen; i += kBlock) {
+            const float x = tile[i];
+            out[i] = apply_scale ? x * scale : x;
+        }
+    }
+}
+
+}  // namespace
+}  // namespace mcclhip
+
+using namespace mcclhip;
+
+extern "C" {
+
+int mccl_hip_topk_decompress(const void* wire, uint64_t wire_bytes, float* dense, uint64_t count,
+                             int* status, void* stream) {
+    if (!wire || (!dense && count) || ((uintptr_t)wire & 3)) return MCCL_HIP_ERR_ARG;
+    if (count > 0xFFFFFFFFull) return MCCL_HIP_ERR_ARG;
+    if (wire_bytes < 4 || ((wire_bytes - 4) & 7)) return MCCL_HIP_ERR_SIZE;
+    const uint64_t k64 = (wire_bytes - 4) / 8;
+    if (k64 > 0xFFFFFFFFull) return MCCL_HIP_ERR_SIZE;
+    int rc = mccl_hip_init();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const uint64_t cap = (uint64_t)device_info().num_cus * (uint64_t)tuning().fold_blocks_per_cu;
+    if (count) {
+        k_fill_zero<<<clamp_u32((count / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(dense, count);
+    }
+    k_scatter<<<clamp_u32((k64 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(
+        (const uint32_t*)wire, (uint32_t)k64, dense, count, status);
+    return launch_status();
+}
+
+int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems,
+                               const void* const* host_wires, int ws, uint64_t wire_stride,
+                               int apply_scale, float scale, int* status, void* stream) {
+    if (!acc || !host_wires || ws < 1 || ws > MCCL_HIP_MAX_WORLD) return MCCL_HIP_ERR_ARG;
+    if (n_total == 0 || n_total > MCCL_HIP_MAX_ELEMS || bucket_elems == 0) return MCCL_HIP_ERR_ARG;
+    if (wire_stride < 4 || (wire_stride & 3)) return MCCL_HIP_ERR_ARG;
+    if (bucket_elems > n_total) bucket_elems = n_total;
+    if (bucket_elems > 0xFFFFFFFFull) return MCCL_HIP_ERR_ARG;
+    const uint64_t nb = (n_total + bucket_elems - 1) / bucket_elems;
+    if (nb > 65535) return MCCL_HIP_ERR_ARG;
+    WirePtrs wp;
+    for (int r = 0; r < MCCL_HIP_MAX_WORLD; r++) wp.w[r] = nullptr;
+    for (int r = 0; r < ws; r++) {
+        if (!host_wires[r] || ((uintptr_t)host_wires[r] & 3)) return MCCL_HIP_ERR_ARG;
+        wp.w[r] = (const uint8_t*)host_wires[r];
+    }
+    int rc = mccl_hip_init();
+    if (rc) return rc;
+    const uint32_t tiles = (uint32_t)((bucket_elems + kAccTile - 1) / kAccTile);
+    k_sparse_accumulate<<<dim3(tiles, (uint32_t)nb), kBlock, 0, (hipStream_t)stream>>>(
+        acc, n_total, bucket_elems, wp, ws, wire_stride, apply_scale, scale, status);
+    return launch_status();
+}
+
+}  // extern "C"

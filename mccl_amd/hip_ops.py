@@ -1,0 +1,173 @@
+"""Tensor-level calls into the C ABI (``include/mccl_hip.h``).
+
+Every function takes ROCm torch tensors, passes ``data_ptr()`` and torch's
+current HIP stream to the library, and only enqueues work.  Nothing here
+computes on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+
+SUM, AVG, PRODUCT, MIN, MAX = 0, 1, 2, 3, 4
+RING_BASIC, RING_CHUNKED = 0, 1
+
+# at::ScalarType values
+_DTYPE_CODE = {
+    torch.uint8: 0, torch.int32: 3, torch.int64: 4, torch.float16: 5,
+    torch.float32: 6, torch.bool: 11, torch.bfloat16: 15,
+}
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise _lib.MCCLHipError(-2, f"dtype {t.dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{what} must live on the GPU, got {t.device}")
+    if not t.is_contiguous():
+        raise ValueError(f"{what} must be contiguous")
+
+
+def fold2(dst: torch.Tensor, src: torch.Tensor, op: int = SUM) -> torch.Tensor:
+    _dev(dst, "dst"); _dev(src, "src")
+    if dst.shape != src.shape or dst.dtype != src.dtype:
+        raise ValueError("shape / dtype mismatch")
+    rc = _lib.load().mccl_hip_fold2(dst.data_ptr(), src.data_ptr(), dst.numel(), dtype_code(dst), op, _stream())
+    _lib.check(rc, "fold2")
+    return dst
+
+
+def scale(buf: torch.Tensor, s: float) -> torch.Tensor:
+    _dev(buf, "buf")
+    rc = _lib.load().mccl_hip_scale(buf.data_ptr(), buf.numel(), dtype_code(buf), s, _stream())
+    _lib.check(rc, "scale")
+    return buf
+
+
+def fold2_scale(dst: torch.Tensor, src: torch.Tensor, s: float) -> torch.Tensor:
+    _dev(dst, "dst"); _dev(src, "src")
+    if dst.shape != src.shape or dst.dtype != src.dtype:
+        raise ValueError("shape / dtype mismatch")
+    rc = _lib.load().mccl_hip_fold2_scale(dst.data_ptr(), src.data_ptr(), dst.numel(), dtype_code(dst), s, _stream())
+    _lib.check(rc, "fold2_scale")
+    return dst
+
+
+def _ptrs(tensors: Sequence[torch.Tensor]):
+    return (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def ring_fold(out: torch.Tensor, ins: Sequence[torch.Tensor], op: int = SUM,
+              schedule: int = RING_BASIC, bucket_elems: Optional[int] = None,
+              scale_by: Optional[float] = None, stepwise: bool = False) -> torch.Tensor:
+    _dev(out, "out")
+    for t in ins:
+        _dev(t, "in")
+        if t.numel() != out.numel() or t.dtype != out.dtype:
+            raise ValueError("shape / dtype mismatch")
+    n = out.numel()
+    rc = _lib.load().mccl_hip_ring_fold(
+        out.data_ptr(), _ptrs(ins), len(ins), n, bucket_elems or max(n, 1), schedule, dtype_code(out), op,
+        0 if scale_by is None else 1, 0.0 if scale_by is None else scale_by, int(stepwise), _stream())
+    _lib.check(rc, "ring_fold")
+    return out
+
+
+def topk_k(count: int, ratio: float) -> int:
+    return int(_lib.load().mccl_hip_topk_k(count, ratio))
+
+
+def topk_max_compressed_size(nbytes: int, ratio: float) -> int:
+    return int(_lib.load().mccl_hip_topk_max_compressed_size(nbytes, ratio))
+
+
+def topk_wire_stride(bucket_elems: int, ratio: float) -> int:
+    """Bytes reserved per bucket payload: the reference's max_compressed_size."""
+    return topk_max_compressed_size(bucket_elems * 4, ratio)
+
+
+def topk_workspace(n_total: int, bucket_elems: int, device) -> torch.Tensor:
+    nbytes = int(_lib.load().mccl_hip_topk_workspace_bytes(n_total, bucket_elems))
+    if nbytes == 0:
+        raise _lib.MCCLHipError(-6, "topk_workspace_bytes")
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
+                  bucket_elems: Optional[int] = None, wire: Optional[torch.Tensor] = None,
+                  workspace: Optional[torch.Tensor] = None, wire_stride: Optional[int] = None):
+    """Returns (wire uint8 tensor [nbuckets * stride], stride). residual is updated."""
+    _dev(grad, "grad"); _dev(residual, "residual")
+    if grad.dtype != torch.float32 or residual.dtype != torch.float32:
+        raise _lib.MCCLHipError(-2, "TopK compression currently supports float32 only")
+    n = grad.numel()
+    be = min(bucket_elems or n, n) if n else 1
+    stride = wire_stride if wire_stride is not None else topk_wire_stride(be, ratio)
+    nb = (n + be - 1) // be if n else 1
+    if wire is None:
+        wire = torch.empty(nb * stride, dtype=torch.uint8, device=grad.device)
+    if workspace is None:
+        workspace = topk_workspace(max(n, 1), be, grad.device)
+    rc = _lib.load().mccl_hip_topk_compress(grad.data_ptr(), residual.data_ptr(), n, be, ratio,
+                                           wire.data_ptr(), stride, workspace.data_ptr(),
+                                           workspace.numel(), _stream())
+    _lib.check(rc, "topk_compress")
+    return wire, stride
+
+
+def topk_decompress(wire: torch.Tensor, wire_bytes: int, count: int,
+                    dense: Optional[torch.Tensor] = None, status: Optional[torch.Tensor] = None):
+    _dev(wire, "wire")
+    if dense is None:
+        dense = torch.empty(count, dtype=torch.float32, device=wire.device)
+    rc = _lib.load().mccl_hip_topk_decompress(wire.data_ptr(), wire_bytes, dense.data_ptr(), count,
+                                             None if status is None else status.data_ptr(), _stream())
+    _lib.check(rc, "topk_decompress")
+    return dense
+
+
+def sparse_accumulate(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_stride: int,
+                      bucket_elems: Optional[int] = None, scale_by: Optional[float] = None,
+                      status: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(acc, "acc")
+    n = acc.numel()
+    rc = _lib.load().mccl_hip_sparse_accumulate(
+        acc.data_ptr(), n, bucket_elems or max(n, 1), _ptrs(wires), len(wires), wire_stride,
+        0 if scale_by is None else 1, 0.0 if scale_by is None else scale_by,
+        None if status is None else status.data_ptr(), _stream())
+    _lib.check(rc, "sparse_accumulate")
+    return acc
+
+
+def fence_signal() -> int:
+    t = C.c_uint64(0)
+    _lib.check(_lib.load().mccl_hip_fence_signal(_stream(), C.byref(t)), "fence_signal")
+    return int(t.value)
+
+
+def fence_wait(ticket: int, timeout_ms: int = 0) -> None:
+    _lib.check(_lib.load().mccl_hip_fence_wait(ticket, timeout_ms), "fence_wait")
+
+
+def fence_query(ticket: int) -> bool:
+    rc = _lib.load().mccl_hip_fence_query(ticket)
+    if rc < 0:
+        raise _lib.MCCLHipError(rc, "fence_query")
+    return bool(rc)
+
+
+def set_tuning(key: str, value: int) -> None:
+    _lib.check(_lib.load().mccl_hip_set_tuning(key.encode(), value), f"set_tuning({key})")

@@ -1,0 +1,195 @@
+"""Top-k compress / decompress / sparse accumulate on the GPU vs the oracle:
+wire bytes and residual bits must be identical (ties -> lower index)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests._gpu_util import DEV, to_dev, to_np, bits, student_t
+
+pytestmark = pytest.mark.gpu
+F32 = oracle.F32
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from mccl_amd import hip_ops
+    return hip_ops
+
+
+def oracle_buckets(g, r, ratio, be):
+    """Per-bucket oracle compress; returns (list of wire arrays, new residual)."""
+    n = g.size
+    res = r.copy()
+    wires = []
+    for s in range(0, n, be):
+        e = min(n, s + be)
+        sub = res[s:e].copy()
+        w, rc = oracle.topk_compress(g[s:e].copy(), sub, ratio)
+        assert rc > 0
+        res[s:e] = sub
+        wires.append(w)
+    return wires, res
+
+
+def check_compress(ops, g, r, ratio, be=None, pad=0):
+    n = g.size
+    be = be or n
+    want_wires, want_res = oracle_buckets(g, r, ratio, be)
+    dg = to_dev(g, F32, pad); dr = to_dev(r, F32, pad)
+    wire, stride = ops.topk_compress(dg, dr, ratio, bucket_elems=be)
+    torch.cuda.synchronize()
+    got_res = to_np(dr, F32)
+    assert np.array_equal(bits(got_res), bits(want_res))
+    assert np.array_equal(to_np(dg, F32), g)  # gradient untouched
+    w = wire.cpu().numpy()
+    for b, ww in enumerate(want_wires):
+        got = w[b * stride: b * stride + ww.size]
+        assert got.tobytes() == ww.tobytes(), f"bucket {b}"
+    return wire, stride, want_wires
+
+
+@pytest.mark.parametrize("n,ratio", [(1, 0.01), (2, 1.0), (99, 0.01), (100, 0.01), (101, 0.5), (4095, 0.01),
+                                     (4096, 0.01), (4097, 0.1), (65_537, 0.01), (300_001, 0.01),
+                                     (300_001, 0.25), (1000, 1.0)])
+def test_compress_single_bucket(ops, n, ratio):
+    rng = np.random.default_rng(n)
+    g = student_t(rng, n, ties=0.01)
+    r = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    check_compress(ops, g, r, ratio)
+    check_compress(ops, g, np.zeros(n, np.float32), ratio, pad=1)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_compress_heavy_ties(ops, seed):
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(1, 200_000))
+    ratio = float(rng.choice([0.001, 0.01, 0.1, 0.5, 1.0]))
+    g = rng.choice(np.array([0.0, -0.0, 0.5, -0.5, 1.0, -1.0, 2.0, 3.0], np.float32), n)
+    r = rng.choice(np.array([0.0, 0.5, -0.5, 1.0], np.float32), n)
+    check_compress(ops, g, r, ratio)
+
+
+def test_compress_degenerate_inputs(ops):
+    n = 50_000
+    check_compress(ops, np.zeros(n, np.float32), np.zeros(n, np.float32), 0.01)        # all equal: pure tie-break
+    check_compress(ops, np.full(n, -2.5, np.float32), np.zeros(n, np.float32), 0.1)
+    g = np.zeros(n, np.float32); g[n - 1] = 1.0; g[0] = -1.0
+    check_compress(ops, g, np.zeros(n, np.float32), 2 / n)
+    big = np.array([3e38, -3e38, 1e-45, -1e-45, np.inf, 0.0, 1.0], np.float32)
+    check_compress(ops, np.tile(big, 1000), np.zeros(7000, np.float32), 0.3)
+
+
+def test_compress_many_buckets_short_last(ops):
+    rng = np.random.default_rng(8)
+    n, be = 1_000_003, 131_072
+    g = student_t(rng, n, ties=0.01)
+    r = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    check_compress(ops, g, r, 0.01, be=be)
+    check_compress(ops, g, r, 0.01, be=be + 1, pad=3)  # buckets at odd element offsets
+
+
+def test_config4_full_bucket_and_error_feedback_over_steps(ops):
+    # one 25 MiB bucket, Student-t nu=3 x 1e-3 with 1 % exact duplicates, k = 65,536
+    n = 6_553_600
+    rng = np.random.default_rng(2024)
+    res_o = np.zeros(n, np.float32)
+    dres = to_dev(res_o, F32)
+    ws = ops.topk_workspace(n, n, DEV)
+    for step in range(2):
+        g = student_t(rng, n, ties=0.01)
+        w, rc = oracle.topk_compress(g, res_o, 0.01)
+        wire, stride = ops.topk_compress(to_dev(g, F32), dres, 0.01, workspace=ws)
+        assert wire.cpu().numpy()[:rc].tobytes() == w.tobytes(), step
+        assert np.array_equal(bits(to_np(dres, F32)), bits(res_o)), step
+    assert oracle.parse_wire(w)[0] == 65_536
+
+
+def test_compress_argument_errors(ops):
+    from mccl_amd._lib import MCCLHipError
+    g = torch.zeros(1000, device=DEV); r = torch.zeros(1000, device=DEV)
+    with pytest.raises(MCCLHipError, match="buffer too small"):
+        ops.topk_compress(g, r, 0.1, wire_stride=4 + 8 * 100 - 4)
+    with pytest.raises(MCCLHipError):
+        ops.topk_compress(g, r, 0.0)
+    with pytest.raises(MCCLHipError):
+        ops.topk_compress(g, r, 1.5)
+    with pytest.raises(MCCLHipError, match="float32 only"):
+        ops.topk_compress(g.half(), r.half(), 0.1)
+    with pytest.raises(MCCLHipError, match="workspace"):
+        ops.topk_compress(g, r, 0.1, workspace=torch.empty(16, dtype=torch.uint8, device=DEV))
+
+
+def test_decompress_matches_oracle_and_reports_errors(ops):
+    rng = np.random.default_rng(5)
+    n = 200_003
+    g = student_t(rng, n)
+    w, rc = oracle.topk_compress(g, np.zeros(n, np.float32), 0.01)
+    want, _ = oracle.topk_decompress(w, n)
+    dw = torch.from_numpy(w).to(DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    dense = torch.full((n + 1,), 7.0, device=DEV)[1:]  # stale contents, misaligned
+    ops.topk_decompress(dw, rc, n, dense=dense, status=status)
+    assert np.array_equal(bits(to_np(dense, F32)), bits(want)) and int(status) == 0
+    # index out of bounds: count == largest index
+    idx_max = int(oracle.parse_wire(w)[1].max())
+    ops.topk_decompress(dw, rc, idx_max, dense=dense[:idx_max], status=status)
+    assert int(status) == oracle.ERR_INDEX
+    # size mismatch: the size that arrived disagrees with the stored k
+    status.zero_()
+    ops.topk_decompress(dw, rc - 8, n, dense=dense, status=status)
+    assert int(status) == oracle.ERR_SIZE
+    from mccl_amd._lib import MCCLHipError
+    with pytest.raises(MCCLHipError, match="size mismatch"):
+        ops.topk_decompress(dw, rc - 3, n, dense=dense, status=status)
+
+
+@pytest.mark.parametrize("ws,n,be", [(8, 300_007, 65_536), (3, 4096, 4096), (2, 5, 5), (8, 1_000_000, 1_000_000)])
+def test_sparse_accumulate_matches_dense_reference_form(ops, ws, n, be):
+    rng = np.random.default_rng(ws + n)
+    ratio = 0.01 if n > 1000 else 0.5
+    nb = (n + be - 1) // be
+    stride = ops.topk_wire_stride(be, ratio)
+    # ~30 % of a rank's picks shared with other ranks: a common pool of large entries
+    shared = rng.random(n) < 0.004
+    dev_wires, per_bucket = [], [[] for _ in range(nb)]
+    for r in range(ws):
+        g = student_t(rng, n, ties=0.0)
+        g[shared] *= 50.0
+        buf = np.zeros(nb * stride, np.uint8)
+        for b in range(nb):
+            s, e = b * be, min(n, (b + 1) * be)
+            w, rc = oracle.topk_compress(g[s:e].copy(), np.zeros(e - s, np.float32), ratio)
+            buf[b * stride: b * stride + rc] = w
+            per_bucket[b].append(w)
+        dev_wires.append(torch.from_numpy(buf).to(DEV))
+    want = np.empty(n, np.float32)
+    for b in range(nb):
+        s, e = b * be, min(n, (b + 1) * be)
+        acc, rc = oracle.sparse_accumulate(per_bucket[b], e - s, scale_by=1.0 / ws)
+        assert rc == oracle.OK
+        want[s:e] = acc
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    acc = torch.full((n,), 3.0, device=DEV)
+    ops.sparse_accumulate(acc, dev_wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status)
+    assert int(status) == 0
+    assert np.array_equal(bits(to_np(acc, F32)), bits(want))
+
+
+def test_sparse_accumulate_flags_bad_payloads(ops):
+    n = 10_000
+    stride = 4 + 8 * 16
+    good = np.zeros(stride, np.uint8)
+    good[:4] = np.array([2], "<u4").view(np.uint8)
+    good[4:20] = np.array([5, 0x3F800000, 9_999, 0x40000000], "<u4").view(np.uint8)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    acc = torch.empty(n, device=DEV)
+    ops.sparse_accumulate(acc, [torch.from_numpy(good).to(DEV)], stride, status=status)
+    assert int(status) == 0 and float(acc[5]) == 1.0 and float(acc[9_999]) == 2.0 and float(acc.sum()) == 3.0
+    bad = good.copy(); bad[12:16] = np.array([10_000], "<u4").view(np.uint8)   # index == count
+    ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status)
+    assert int(status) == oracle.ERR_INDEX
+    status.zero_()
+    bad = good.copy(); bad[:4] = np.array([17], "<u4").view(np.uint8)           # k beyond the stride
+    ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status)
+    assert int(status) == oracle.ERR_SIZE
