@@ -1,0 +1,293 @@
+#!/usr/bin/env python3
+"""Throughput of the per-rank data-parallel compute path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only fold|all]
+
+A "step" is one pass of the hot path over one batch of synthetic input with the
+inputs already resident in HBM: the fp32 ring reduce-scatter fold of a
+96,510,024-element gradient held by 8 simulated ranks (25 MiB buckets, 8 chunks
+per bucket, 7 folds per chunk slot in ring-step order, then AVG x 1/8).  The one
+JSON line printed at the end carries that figure as `value`, its roofline
+block, the CPU baseline timed on this box's host cores, and (under `extra`) the
+other workloads of the path: the binary fold of one bucket, the step-wise
+drop-in sequence, the bf16/fp16 folds, top-k 1 % compression and the
+decompress-accumulate.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N_GRAD = 96_510_024          # HeavyDummyModel parameter count of the reference
+BUCKET = 6_553_600           # 25 MiB of fp32: DDP's default bucket
+HBM_PEAK_GBPS = 8000.0       # MI355X published HBM3E peak
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="all", choices=["all", "fold"],
+                    help="fold: only the headline workload (used for profiling runs)")
+    ap.add_argument("--elems", type=int, default=N_GRAD, help="gradient elements (default: the full 96.5 M)")
+    return ap.parse_args()
+
+
+def main() -> int:
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: every rank's buffer lives in that GPU's HBM and nothing "
+              "here uses a second device; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    from mccl_amd import hip_ops as ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    N = a.elems
+    W = 8
+    K, WU = a.steps, a.warmup
+
+    def gpu_time(fn, steps=K, warmup=WU):
+        """Returns (wall ms per step, list of per-launch-group event ms)."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        t0 = time.perf_counter()
+        for s, e in evs:
+            s.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return wall, [s.elapsed_time(e) for s, e in evs]
+
+    def stats(ms_list):
+        arr = sorted(ms_list)
+        return {"avg_ms": sum(arr) / len(arr), "median_ms": arr[len(arr) // 2], "min_ms": arr[0]}
+
+    def rate(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9
+
+    extra = {}
+
+    # ---- config 2: the headline workload -----------------------------------
+    gens = [torch.Generator(device=dev).manual_seed(1000 + r) for r in range(W)]
+    ranks = [torch.randn(N, generator=gens[r], device=dev).mul_(1e-3) for r in range(W)]
+    out = torch.empty(N, device=dev)
+    fold_bytes = (W + 1) * 4 * N
+
+    def step_fold():
+        ops.ring_fold(out, ranks, ops.AVG, ops.RING_BASIC, bucket_elems=BUCKET, scale_by=0.125)
+
+    wall_ms, ev_ms = gpu_time(step_fold)
+    st = stats(ev_ms)
+    fold_gbps = rate(fold_bytes, wall_ms)
+    roofline = {
+        "bound": "hbm", "kernel": "k_ring_fold<f32,add>",
+        "achieved": rate(fold_bytes, st["avg_ms"]), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": rate(fold_bytes, st["avg_ms"]) / HBM_PEAK_GBPS, "traffic": None,
+        "bytes_per_launch": fold_bytes, "avg_launch_ms": st["avg_ms"], "min_launch_ms": st["min_ms"],
+    }
+
+    # device-to-device copy ceiling with the same timing method (read N, write N)
+    cpy_ms = stats(gpu_time(lambda: out.copy_(ranks[0]))[1])
+    extra["d2d_copy_GBps"] = rate(8 * N, cpy_ms["avg_ms"])
+
+    if a.only == "all":
+        # ---- step-wise drop-in sequence: 7 binary folds per chunk view + scale --
+        work = [r.clone() for r in ranks[:2]]  # only shapes matter for timing; reuse two buffers
+        nb = (N + BUCKET - 1) // BUCKET
+
+        def step_stepwise():
+            for b in range(nb):
+                lo, hi = b * BUCKET, min(N, (b + 1) * BUCKET)
+                ce = (hi - lo + W - 1) // W
+                for c in range(W):
+                    s, e = lo + c * ce, min(hi, lo + (c + 1) * ce)
+                    if s >= e:
+                        continue
+                    for j in range(1, W):
+                        ops.fold2(out[s:e], ranks[(c + j) % W][s:e], ops.SUM)
+                ops.scale(out[lo:hi], 0.125)
+
+        sw = stats(gpu_time(step_stepwise, steps=max(2, K // 5), warmup=1)[1])
+        extra["stepwise_dropin"] = {"ms": sw["avg_ms"], "GBps": rate((12 * (W - 1) + 8) * N, sw["avg_ms"]),
+                                    "bytes_per_elem": 12 * (W - 1) + 8, "launches": nb * (W * (W - 1) + 1)}
+
+        # ---- config 1: one 25 MiB bucket, W=2, fused (x0 + x1) * 0.5 ------------
+        b0, b1 = ranks[0][:BUCKET].clone(), ranks[1][:BUCKET].clone()
+        c1 = stats(gpu_time(lambda: ops.fold2_scale(b0, b1, 0.5))[1])
+        extra["config1_fold2_scale_bucket"] = {"ms": c1["avg_ms"], "GBps": rate(12 * BUCKET, c1["avg_ms"]),
+                                               "note": "78.6 MB working set: Infinity-Cache resident"}
+        # same kernel over the whole gradient: HBM-resident figure
+        c1w = stats(gpu_time(lambda: ops.fold2_scale(work[0], work[1], 0.5))[1])
+        extra["fold2_scale_whole_gradient"] = {"ms": c1w["avg_ms"], "GBps": rate(12 * N, c1w["avg_ms"]),
+                                               "frac": rate(12 * N, c1w["avg_ms"]) / HBM_PEAK_GBPS}
+        c1f = stats(gpu_time(lambda: ops.fold2(work[0], work[1], ops.SUM))[1])
+        extra["fold2_whole_gradient"] = {"ms": c1f["avg_ms"], "GBps": rate(12 * N, c1f["avg_ms"]),
+                                         "frac": rate(12 * N, c1f["avg_ms"]) / HBM_PEAK_GBPS}
+        del work, b0, b1
+
+        # ---- config 3: bf16 / fp16, W = 4, SUM (+ x0.25) and MAX ----------------
+        for name, tdt in (("bf16", torch.bfloat16), ("fp16", torch.float16)):
+            hs = []
+            for r in range(4):
+                x = torch.randn(N, generator=gens[r], device=dev).mul_(1e-3)
+                m = torch.rand(N, generator=gens[r], device=dev) < 1e-3
+                x[m] *= 1e3
+                hs.append(x.to(tdt))
+                del x, m
+            ho = torch.empty(N, device=dev, dtype=tdt)
+            res = {}
+            for label, kw in (("sum_avg_single_rounding", dict(op=ops.AVG, scale_by=0.25, stepwise=False)),
+                              ("sum_avg_stepwise", dict(op=ops.AVG, scale_by=0.25, stepwise=True)),
+                              ("max", dict(op=ops.MAX))):
+                s3 = stats(gpu_time(lambda: ops.ring_fold(ho, hs, schedule=ops.RING_BASIC,
+                                                          bucket_elems=2 * BUCKET, **kw))[1])
+                res[label] = {"ms": s3["avg_ms"], "GBps": rate(10 * N, s3["avg_ms"]),
+                              "frac": rate(10 * N, s3["avg_ms"]) / HBM_PEAK_GBPS}
+            extra[f"config3_{name}_w4"] = res
+            del hs, ho
+
+        # ---- config 4: top-k 1 % with error feedback, per 25 MiB bucket ----------
+        g = torch.randn(N, generator=gens[0], device=dev)
+        chi = sum(torch.randn(N, generator=gens[1], device=dev).square_() for _ in range(3)).div_(3).sqrt_()
+        grad = g.div_(chi).mul_(1e-3)
+        del chi
+        m = N // 100
+        dst = torch.randint(0, N, (m,), generator=gens[2], device=dev)
+        src = torch.randint(0, N, (m,), generator=gens[2], device=dev)
+        sign = torch.where(torch.rand(m, generator=gens[2], device=dev) < 0.5, -1.0, 1.0)
+        grad[dst] = grad[src] * sign
+        residual0 = torch.randn(N, generator=gens[3], device=dev).mul_(1e-4)
+        residual = residual0.clone()
+        stride = ops.topk_wire_stride(BUCKET, 0.01)
+        nb = (N + BUCKET - 1) // BUCKET
+        wire = torch.empty(nb * stride, dtype=torch.uint8, device=dev)
+        wsb = ops.topk_workspace(N, BUCKET, dev)
+        ks = [ops.topk_k(min(BUCKET, N - b * BUCKET), 0.01) for b in range(nb)]
+        topk_bytes = 12 * N + sum(8 * k + 4 for k in ks)
+
+        def step_topk():
+            ops.topk_compress(grad, residual, 0.01, bucket_elems=BUCKET, wire=wire, workspace=wsb,
+                              wire_stride=stride)
+
+        tk = stats(gpu_time(step_topk)[1])
+        extra["config4_topk_compress"] = {"ms": tk["avg_ms"], "GBps": rate(topk_bytes, tk["avg_ms"]),
+                                          "frac": rate(topk_bytes, tk["avg_ms"]) / HBM_PEAK_GBPS,
+                                          "elems_per_s": N / (tk["avg_ms"] * 1e-3),
+                                          "bytes": topk_bytes, "buckets": nb, "k_per_bucket": ks[0]}
+        # one bucket alone (the reference's call granularity; cache resident)
+        r1 = residual0[:BUCKET].clone()
+        ws1 = ops.topk_workspace(BUCKET, BUCKET, dev)
+        w1 = torch.empty(stride, dtype=torch.uint8, device=dev)
+        tb = stats(gpu_time(lambda: ops.topk_compress(grad[:BUCKET], r1, 0.01, wire=w1, workspace=ws1,
+                                                      wire_stride=stride))[1])
+        extra["config4_topk_one_bucket"] = {"ms": tb["avg_ms"],
+                                            "GBps": rate(12 * BUCKET + 8 * ks[0] + 4, tb["avg_ms"])}
+
+        # ---- config 5: decompress-accumulate of 8 ranks' payloads -----------------
+        shared = torch.rand(N, generator=gens[4], device=dev) < 0.004
+        wires = []
+        for r in range(W):
+            gr = torch.randn(N, generator=gens[r], device=dev).mul_(1e-2)
+            gr[shared] *= 50.0
+            rz = torch.zeros(N, device=dev)
+            wr = torch.empty(nb * stride, dtype=torch.uint8, device=dev)
+            ops.topk_compress(gr, rz, 0.01, bucket_elems=BUCKET, wire=wr, workspace=wsb, wire_stride=stride)
+            wires.append(wr)
+            del gr, rz
+        status = torch.zeros(1, dtype=torch.int32, device=dev)
+        acc = torch.empty(N, device=dev)
+        acc_bytes = 4 * N + 8 * sum(ks) * W
+        sa = stats(gpu_time(lambda: ops.sparse_accumulate(acc, wires, stride, bucket_elems=BUCKET,
+                                                          scale_by=0.125, status=status))[1])
+        extra["config5_sparse_accumulate"] = {"ms": sa["avg_ms"], "GBps": rate(acc_bytes, sa["avg_ms"]),
+                                              "frac": rate(acc_bytes, sa["avg_ms"]) / HBM_PEAK_GBPS,
+                                              "bytes": acc_bytes, "status": int(status)}
+
+    # ---- CPU baseline: the reference's CPU fold path restated, same workload ----
+    cpu = None
+    if not a.no_cpu:
+        import oracle
+        nbk = min(2, (N + BUCKET - 1) // BUCKET)     # bounded sample: 2 buckets of the 15
+        cn = min(N, nbk * BUCKET)
+        host = [r[:cn].cpu().numpy() for r in ranks]
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            for b in range(nbk):
+                lo, hi = b * BUCKET, min(cn, (b + 1) * BUCKET)
+                ce = (hi - lo + W - 1) // W
+                acc_np = np.empty(hi - lo, np.float32)
+                for c in range(W):
+                    s, e = lo + c * ce, min(hi, lo + (c + 1) * ce)
+                    if s >= e:
+                        continue
+                    part = host[c][s:e].copy()
+                    for j in range(1, W):
+                        local = host[(c + j) % W][s:e].copy()
+                        oracle.fold2(local, part, oracle.F32, oracle.OP_SUM, threads=0)  # reference job split
+                        part = local
+                    acc_np[s - lo:e - lo] = part
+                oracle.scale(acc_np, oracle.F32, 0.125, threads=0)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 8:
+                break
+        cpu_s = (time.perf_counter() - t0) / reps
+        cpu = {"value": (W + 1) * 4 * cn / cpu_s / 1e9, "unit": "GB/s", "cores": min(8, os.cpu_count() or 1),
+               "kind": "port",
+               "sample": f"{nbk} of {(N + BUCKET - 1) // BUCKET} buckets ({cn} elements), {reps} repetitions; "
+                         "step-wise ring folds with the reference's job split (>= 1 Mi floats per job, <= 8 jobs), "
+                         "same 36 B/element numerator",
+               "host_cores_visible": os.cpu_count()}
+        if a.only == "all" and oracle.RefCompressor.available():
+            ref = oracle.RefCompressor(2, 0.01)
+            gh = grad[:BUCKET].cpu().numpy()
+            ref.compress(gh, stable_id=1)
+            t0 = time.perf_counter()
+            reps = 0
+            while time.perf_counter() - t0 < 8.0 and reps < 6:
+                ref.compress(gh, stable_id=1)
+                reps += 1
+            s_ref = (time.perf_counter() - t0) / reps
+            extra["config4_cpu_reference_topk"] = {
+                "GBps": (12 * BUCKET + 8 * 65_536 + 4) / s_ref / 1e9, "ms_per_bucket": s_ref * 1e3,
+                "cores": 1, "kind": "reference",
+                "sample": f"one 25 MiB bucket, {reps} repetitions of the reference's compiled TopKCompressor::compress"}
+
+    line = {
+        "metric": "HBM GB/s (% of peak) for fp32 bucket fold and top-k 1% compress, 1 GPU",
+        "value": fold_gbps, "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": WU,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: fp32 ring reduce-scatter fold, 8 simulated ranks in one GPU's HBM, "
+                               f"{N}-element gradient, 25 MiB buckets x 8 chunks, 7 folds per chunk slot in "
+                               "ring-step order, AVG x 1/8 fused",
+                   "elements": N, "world_size": W, "bucket_elems": BUCKET, "bytes_per_element": 36,
+                   "elements_per_s": N / (wall_ms * 1e-3), "pct_of_hbm_peak": 100.0 * fold_gbps / HBM_PEAK_GBPS},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -47,6 +47,12 @@ def load() -> C.CDLL:
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build it with `python -m mccl_amd.build --lib` "
                 "(there is no CPU fallback for the HIP kernels)")
+        try:
+            # torch ships its own HIP runtime under the same soname; load it
+            # first so the process ends up with exactly one runtime
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)

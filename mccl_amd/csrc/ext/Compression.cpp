@@ -1,0 +1,117 @@
+#include "Compression.hpp"
+
+#include <c10/hip/HIPStream.h>
+
+#include "../../../include/mccl_hip.h"
+#include "Errors.hpp"
+#include "HipKernels.hpp"
+#include "Logging.hpp"
+#include "TopKCompression.hpp"
+
+namespace mccl {
+
+std::unique_ptr<Compressor> make_compressor(CompressionMode mode, double param) {
+    switch (mode) {
+        case CompressionMode::NONE: return nullptr;
+        case CompressionMode::TOPK: return std::make_unique<TopKCompressor>(param > 0 ? param : 0.01);
+        default:
+            throw MCCLError("Unknown compression mode: " + std::to_string(static_cast<int>(mode)));
+    }
+}
+
+TopKCompressor::TopKCompressor(double k_ratio) : k_ratio_(k_ratio) {
+    MCCL_CHECK(k_ratio > 0 && k_ratio <= 1.0, "k_ratio must be in (0, 1], got " + std::to_string(k_ratio));
+}
+
+// csrc/compression/TopKCompression.cpp:38-120.  The residual map keeps the
+// reference's rules: a new id while 1024 ids are live clears the map (:57-62);
+// an id whose element count changed starts again from zeros (:63-66).
+size_t TopKCompressor::compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
+                                at::ScalarType dtype, uint64_t stable_id) {
+    MCCL_CHECK(dtype == at::kFloat, "TopK compression currently supports float32 only");
+    const size_t count = nbytes / sizeof(float);
+    MCCL_CHECK(count > 0, "TopK compress: empty input");
+    const uint32_t k = mccl_hip_topk_k(count, k_ratio_);
+    const size_t output_size = sizeof(uint32_t) + static_cast<size_t>(k) * 8;
+    MCCL_CHECK(dst_capacity >= output_size, "TopK compress: buffer too small");
+
+    std::lock_guard<std::mutex> lock(mu_);
+    metal_kernels_init();
+    const auto opts_f = at::TensorOptions().dtype(at::kFloat).device(at::kCUDA);
+    if (error_buffers_.size() >= kMaxErrorBuffers && error_buffers_.find(stable_id) == error_buffers_.end()) {
+        MCCL_WARN("TopK: evicting all %zu error feedback buffers (unstable tensor identities?)",
+                  error_buffers_.size());
+        error_buffers_.clear();
+    }
+    auto it = error_buffers_.find(stable_id);
+    if (it == error_buffers_.end() || static_cast<size_t>(it->second.numel()) != count) {
+        error_buffers_[stable_id] = at::zeros({static_cast<int64_t>(count)}, opts_f);
+    }
+    at::Tensor& residual = error_buffers_[stable_id];
+
+    const uint64_t ws_bytes = mccl_hip_topk_workspace_bytes(count, count);
+    if (!workspace_.defined() || static_cast<uint64_t>(workspace_.numel()) < ws_bytes) {
+        workspace_ = at::empty({static_cast<int64_t>(ws_bytes)},
+                               at::TensorOptions().dtype(at::kByte).device(at::kCUDA));
+    }
+    // The payload's pairs start 4 bytes in; the stride only has to be a multiple of 4.
+    const uint64_t stride = static_cast<uint64_t>(dst_capacity) & ~uint64_t(3);
+    const int rc = mccl_hip_topk_compress(static_cast<const float*>(src), residual.data_ptr<float>(), count,
+                                          count, k_ratio_, dst, stride, workspace_.data_ptr(),
+                                          static_cast<uint64_t>(workspace_.numel()),
+                                          c10::hip::getCurrentHIPStream().stream());
+    if (rc == MCCL_HIP_ERR_CAPACITY) throw MCCLError("TopK compress: buffer too small");
+    throw_on_status(rc, "TopK compress");
+    MCCL_TRACE("TopK compress: %zu elements -> %u values, output %zu bytes", count, k, output_size);
+    return output_size;
+}
+
+// csrc/compression/TopKCompression.cpp:122-152.  The reference validates while
+// it scatters and throws; here the kernel reports through a device flag that
+// is read back once the stream has drained (the call is synchronous, as the
+// reference's is).
+void TopKCompressor::decompress(const void* src, size_t compressed_size, void* dst, size_t nbytes,
+                                at::ScalarType dtype) {
+    MCCL_CHECK(dtype == at::kFloat, "TopK decompression currently supports float32 only");
+    const size_t count = nbytes / sizeof(float);
+    std::lock_guard<std::mutex> lock(mu_);
+    metal_kernels_init();
+    if (!status_.defined()) status_ = at::zeros({1}, at::TensorOptions().dtype(at::kInt).device(at::kCUDA));
+    status_.zero_();
+    const int rc = mccl_hip_topk_decompress(src, compressed_size, static_cast<float*>(dst), count,
+                                            status_.data_ptr<int>(), c10::hip::getCurrentHIPStream().stream());
+    if (rc == MCCL_HIP_ERR_SIZE) throw MCCLError("TopK decompress: size mismatch");
+    throw_on_status(rc, "TopK decompress");
+    const int st = status_.item<int>();
+    if (st == MCCL_HIP_ERR_SIZE) throw MCCLError("TopK decompress: size mismatch");
+    if (st == MCCL_HIP_ERR_INDEX) throw MCCLError("TopK decompress: index out of bounds");
+}
+
+size_t TopKCompressor::max_compressed_size(size_t nbytes) const {
+    return static_cast<size_t>(mccl_hip_topk_max_compressed_size(nbytes, k_ratio_));
+}
+
+void TopKCompressor::reset_error_feedback() {
+    std::lock_guard<std::mutex> lock(mu_);
+    error_buffers_.clear();
+    MCCL_DEBUG("TopK: all error feedback buffers reset");
+}
+
+void TopKCompressor::reset_error_feedback_for_tensor(uint64_t stable_id) {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = error_buffers_.find(stable_id);
+    if (it != error_buffers_.end()) it->second.zero_();
+}
+
+size_t TopKCompressor::error_feedback_buffer_count() const {
+    std::lock_guard<std::mutex> lock(mu_);
+    return error_buffers_.size();
+}
+
+at::Tensor TopKCompressor::error_feedback_buffer(uint64_t stable_id) const {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = error_buffers_.find(stable_id);
+    return it == error_buffers_.end() ? at::Tensor() : it->second;
+}
+
+}  // namespace mccl

@@ -1,0 +1,174 @@
+// pybind module `mccl_amd._C`: the part of the reference's `mccl._C`
+// (csrc/backend/Registration.cpp:220-312) that belongs to the per-rank compute
+// path -- version attributes, CompressionMode, MCCLOptions and the six
+// `_metal_*` kernel helpers with their "init, sync producer, kernel, sync"
+// shape and "returns the same tensor" contract -- plus tensor-level access to
+// the compressor and the ring fold.
+#include <torch/extension.h>
+#include <torch/csrc/utils/pybind.h>
+
+#include <c10/hip/HIPStream.h>
+
+#include "../../../include/mccl_hip.h"
+#include "Compression.hpp"
+#include "Errors.hpp"
+#include "HipKernels.hpp"
+#include "Options.hpp"
+#include "TensorChecks.hpp"
+#include "TopKCompression.hpp"
+
+namespace py = pybind11;
+
+namespace {
+
+// Producer-side sync of the helpers: the reference drains torch's MPS stream
+// before touching the buffers (mps_stream_sync).  The kernels here run on
+// torch's current stream, so ordering is already given; the sync is kept so the
+// helpers stay blocking calls.
+void producer_sync() { mccl::metal_sync(); }
+
+uint64_t stable_id_of(const at::Tensor& t) {
+    // storage address + offset, stable across steps for DDP buckets
+    // (csrc/backend/ProcessGroupMCCL.cpp:1080-1083)
+    return reinterpret_cast<uint64_t>(t.storage().data()) +
+           static_cast<uint64_t>(t.storage_offset()) * t.element_size();
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.attr("__version__") = "0.5.0";
+    m.attr("__protocol_version__") = 5;
+    m.attr("__hip_abi_version__") = mccl_hip_abi_version();
+
+    py::enum_<mccl::CompressionMode>(m, "CompressionMode")
+        .value("NONE", mccl::CompressionMode::NONE)
+        .value("FP16", mccl::CompressionMode::FP16)
+        .value("TOPK", mccl::CompressionMode::TOPK);
+
+    py::class_<mccl::MCCLOptions, c10d::Backend::Options, c10::intrusive_ptr<mccl::MCCLOptions>>(m, "MCCLOptions")
+        .def(py::init<>())
+        .def(py::init<std::chrono::milliseconds>(), py::arg("timeout"))
+        .def_readwrite("transport", &mccl::MCCLOptions::transport)
+        .def_readwrite("listen_addr", &mccl::MCCLOptions::listen_addr)
+        .def_readwrite("port_base", &mccl::MCCLOptions::port_base)
+        .def_readwrite("ifname", &mccl::MCCLOptions::ifname)
+        .def_readwrite("chunk_bytes", &mccl::MCCLOptions::chunk_bytes)
+        .def_readwrite("small_msg_threshold", &mccl::MCCLOptions::small_msg_threshold)
+        .def_readwrite("transport_crc", &mccl::MCCLOptions::transport_crc)
+        .def_readwrite("fast_math", &mccl::MCCLOptions::fast_math)
+        .def_readwrite("gpu_threshold", &mccl::MCCLOptions::gpu_threshold)
+        .def_readwrite("overlap_comm", &mccl::MCCLOptions::overlap_comm)
+        .def_readwrite("max_queue_depth", &mccl::MCCLOptions::max_queue_depth)
+        .def_readwrite("compression", &mccl::MCCLOptions::compression)
+        .def_readwrite("topk_ratio", &mccl::MCCLOptions::topk_ratio)
+        .def_readwrite("watchdog_timeout", &mccl::MCCLOptions::watchdog_timeout)
+        .def_readwrite("heartbeat_interval", &mccl::MCCLOptions::heartbeat_interval);
+
+    // ---- kernel helpers: same names as the reference's test bindings ----------
+    m.def("_metal_accumulate_chunk", [](at::Tensor dst, const at::Tensor& src) {
+        mccl::metal_kernels_init(); producer_sync();
+        mccl::metal_accumulate_chunk(dst, src);
+        mccl::metal_sync();
+        return dst;
+    }, "dst += src via the HIP kernel; returns dst");
+    m.def("_metal_elementwise_min", [](at::Tensor dst, const at::Tensor& src) {
+        mccl::metal_kernels_init(); producer_sync();
+        mccl::metal_elementwise_min(dst, src);
+        mccl::metal_sync();
+        return dst;
+    }, "dst = min(dst, src); returns dst");
+    m.def("_metal_elementwise_max", [](at::Tensor dst, const at::Tensor& src) {
+        mccl::metal_kernels_init(); producer_sync();
+        mccl::metal_elementwise_max(dst, src);
+        mccl::metal_sync();
+        return dst;
+    }, "dst = max(dst, src); returns dst");
+    m.def("_metal_elementwise_product", [](at::Tensor dst, const at::Tensor& src) {
+        mccl::metal_kernels_init(); producer_sync();
+        mccl::metal_elementwise_product(dst, src);
+        mccl::metal_sync();
+        return dst;
+    }, "dst *= src; returns dst");
+    m.def("_metal_scale_inplace", [](at::Tensor buf, double scale) {
+        mccl::metal_kernels_init(); producer_sync();
+        mccl::metal_scale_inplace(buf, scale);
+        mccl::metal_sync();
+        return buf;
+    }, "buf *= scale; returns buf");
+    m.def("_metal_accumulate_and_scale", [](at::Tensor dst, const at::Tensor& src, double scale) {
+        mccl::metal_kernels_init(); producer_sync();
+        mccl::metal_accumulate_and_scale(dst, src, scale);
+        mccl::metal_sync();
+        return dst;
+    }, "dst = (dst + src) * scale; returns dst");
+
+    // ---- the C++ entry points the process group calls, asynchronous ---------
+    m.def("_metal_reduce_op", [](at::Tensor dst, const at::Tensor& src, int op) {
+        mccl::metal_kernels_init();
+        mccl::metal_reduce_op(dst, src, static_cast<c10d::ReduceOp::RedOpType>(op));
+        return dst;
+    });
+    m.def("_metal_reduce_op_fenced", [](at::Tensor dst, const at::Tensor& src, int op) {
+        mccl::metal_kernels_init();
+        return mccl::metal_reduce_op_fenced(dst, src, static_cast<c10d::ReduceOp::RedOpType>(op));
+    });
+    m.def("_wait_for_mccl_fence", &mccl::wait_for_mccl_fence);
+    m.def("_event_sync_available", [] { mccl::event_sync_init(); return mccl::event_sync_available(); });
+    m.def("_metal_sync", &mccl::metal_sync);
+    m.def("_hip_ring_fold", [](at::Tensor out, const std::vector<at::Tensor>& ins, int op, bool chunked,
+                               int64_t bucket_elems, bool stepwise) {
+        mccl::metal_kernels_init();
+        mccl::hip_ring_fold(out, ins, static_cast<c10d::ReduceOp::RedOpType>(op), chunked, bucket_elems, stepwise);
+        return out;
+    }, py::arg("out"), py::arg("ins"), py::arg("op"), py::arg("chunked") = false,
+       py::arg("bucket_elems") = 0, py::arg("stepwise") = false);
+    m.def("_cpu_reduce_op", [](at::Tensor dst, const at::Tensor& src, int op) {
+        // raw-pointer family on device pointers, fp32 only here (test hook)
+        mccl::check_same_shape_dtype(dst, src);
+        MCCL_CHECK(dst.scalar_type() == at::kFloat, "float32 only");
+        mccl::cpu_reduce_op(dst.data_ptr<float>(), src.data_ptr<float>(), dst.numel(),
+                            static_cast<c10d::ReduceOp::RedOpType>(op));
+        return dst;
+    });
+
+    // ---- compressor -------------------------------------------------------------
+    py::class_<mccl::TopKCompressor>(m, "TopKCompressor")
+        .def(py::init<double>(), py::arg("k_ratio"))
+        .def("name", &mccl::TopKCompressor::name)
+        .def("max_compressed_size", &mccl::TopKCompressor::max_compressed_size)
+        .def("compress", [](mccl::TopKCompressor& c, const at::Tensor& t, py::object stable_id, py::object capacity) {
+            mccl::check_single_tensor(t);
+            const size_t nbytes = mccl::tensor_nbytes(t);
+            const size_t cap = capacity.is_none() ? c.max_compressed_size(nbytes) : capacity.cast<size_t>();
+            at::Tensor out = at::empty({static_cast<int64_t>(cap)},
+                                       at::TensorOptions().dtype(at::kByte).device(t.device()));
+            const uint64_t id = stable_id.is_none() ? stable_id_of(t) : stable_id.cast<uint64_t>();
+            const size_t used = c.compress(t.data_ptr(), nbytes, out.data_ptr(), cap, t.scalar_type(), id);
+            return out.narrow(0, 0, static_cast<int64_t>(used));
+        }, py::arg("tensor"), py::arg("stable_id") = py::none(), py::arg("capacity") = py::none(),
+           "Top-k payload of a gradient bucket as a uint8 device tensor; error feedback is kept per stable_id")
+        .def("decompress", [](mccl::TopKCompressor& c, const at::Tensor& wire, int64_t numel, py::object size) {
+            at::Tensor out = at::empty({numel}, at::TensorOptions().dtype(at::kFloat).device(wire.device()));
+            const size_t sz = size.is_none() ? static_cast<size_t>(wire.numel()) : size.cast<size_t>();
+            c.decompress(wire.data_ptr(), sz, out.data_ptr(), static_cast<size_t>(numel) * 4, at::kFloat);
+            return out;
+        }, py::arg("wire"), py::arg("numel"), py::arg("compressed_size") = py::none())
+        .def("reset_error_feedback", &mccl::TopKCompressor::reset_error_feedback)
+        .def("reset_error_feedback_for_tensor", &mccl::TopKCompressor::reset_error_feedback_for_tensor)
+        .def("error_feedback_buffer_count", &mccl::TopKCompressor::error_feedback_buffer_count)
+        .def("error_feedback_buffer", [](mccl::TopKCompressor& c, uint64_t id) -> py::object {
+            at::Tensor t = c.error_feedback_buffer(id);
+            if (!t.defined()) return py::none();
+            return py::cast(t);
+        });
+    m.def("make_compressor", [](mccl::CompressionMode mode, double param) -> py::object {
+        auto c = mccl::make_compressor(mode, param);
+        if (!c) return py::none();
+        auto* topk = dynamic_cast<mccl::TopKCompressor*>(c.get());
+        MCCL_CHECK(topk != nullptr, "unexpected compressor type");
+        c.release();
+        return py::cast(topk, py::return_value_policy::take_ownership);
+    }, py::arg("mode"), py::arg("param") = 0.0);
+    m.def("_compression_stable_id", &stable_id_of);
+}
