@@ -197,7 +197,7 @@ int mccl_hip_fence_block_stream(uint64_t ticket, void* stream);
 int mccl_hip_sync(void* stream);
 
 /* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
-/* keys: "fold_blocks_per_cu", "fold_unroll", "nontemporal", "topk_path"  */
+/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path" */
 int mccl_hip_set_tuning(const char* key, int value);
 int mccl_hip_get_tuning(const char* key);
 

@@ -82,9 +82,6 @@ int mccl_hip_set_tuning(const char* key, int value) {
     if (!std::strcmp(key, "fold_blocks_per_cu")) {
         if (value < 1 || value > 64) return MCCL_HIP_ERR_ARG;
         t.fold_blocks_per_cu = value;
-    } else if (!std::strcmp(key, "fold_unroll")) {
-        if (value != 1 && value != 2 && value != 4) return MCCL_HIP_ERR_ARG;
-        t.fold_unroll = value;
     } else if (!std::strcmp(key, "nontemporal")) {
         t.nontemporal = value ? 1 : 0;
     } else if (!std::strcmp(key, "topk_path")) {
@@ -100,7 +97,6 @@ int mccl_hip_get_tuning(const char* key) {
     if (!key) return MCCL_HIP_ERR_ARG;
     const Tuning& t = tuning();
     if (!std::strcmp(key, "fold_blocks_per_cu")) return t.fold_blocks_per_cu;
-    if (!std::strcmp(key, "fold_unroll")) return t.fold_unroll;
     if (!std::strcmp(key, "nontemporal")) return t.nontemporal;
     if (!std::strcmp(key, "topk_path")) return t.topk_path;
     return MCCL_HIP_ERR_ARG;
