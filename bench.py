@@ -35,8 +35,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="all", choices=["all", "fold"],
-                    help="fold: only the headline workload (used for profiling runs)")
+    ap.add_argument("--only", default="all", choices=["all", "fold", "topk", "sparse"],
+                    help="fold / topk / sparse: the headline workload plus only that part (profiling runs)")
     ap.add_argument("--elems", type=int, default=N_GRAD, help="gradient elements (default: the full 96.5 M)")
     return ap.parse_args()
 
@@ -164,6 +164,7 @@ def main() -> int:
             extra[f"config3_{name}_w4"] = res
             del hs, ho
 
+    if a.only in ("all", "topk", "sparse"):
         # ---- config 4: top-k 1 % with error feedback, per 25 MiB bucket ----------
         g = torch.randn(N, generator=gens[0], device=dev)
         chi = sum(torch.randn(N, generator=gens[1], device=dev).square_() for _ in range(3)).div_(3).sqrt_()
@@ -179,7 +180,7 @@ def main() -> int:
         stride = ops.topk_wire_stride(BUCKET, 0.01)
         nb = (N + BUCKET - 1) // BUCKET
         wire = torch.empty(nb * stride, dtype=torch.uint8, device=dev)
-        wsb = ops.topk_workspace(N, BUCKET, dev)
+        wsb = ops.topk_workspace(N, BUCKET, 0.01, dev)
         ks = [ops.topk_k(min(BUCKET, N - b * BUCKET), 0.01) for b in range(nb)]
         topk_bytes = 12 * N + sum(8 * k + 4 for k in ks)
 
@@ -191,10 +192,11 @@ def main() -> int:
         extra["config4_topk_compress"] = {"ms": tk["avg_ms"], "GBps": rate(topk_bytes, tk["avg_ms"]),
                                           "frac": rate(topk_bytes, tk["avg_ms"]) / HBM_PEAK_GBPS,
                                           "elems_per_s": N / (tk["avg_ms"] * 1e-3),
-                                          "bytes": topk_bytes, "buckets": nb, "k_per_bucket": ks[0]}
+                                          "bytes": topk_bytes, "buckets": nb, "k_per_bucket": ks[0],
+                                          "single_pass_buckets": ops.topk_path_report(wsb, N, BUCKET, 0.01)[0]}
         # one bucket alone (the reference's call granularity; cache resident)
         r1 = residual0[:BUCKET].clone()
-        ws1 = ops.topk_workspace(BUCKET, BUCKET, dev)
+        ws1 = ops.topk_workspace(BUCKET, BUCKET, 0.01, dev)
         w1 = torch.empty(stride, dtype=torch.uint8, device=dev)
         tb = stats(gpu_time(lambda: ops.topk_compress(grad[:BUCKET], r1, 0.01, wire=w1, workspace=ws1,
                                                       wire_stride=stride))[1])
@@ -256,7 +258,7 @@ def main() -> int:
                          "step-wise ring folds with the reference's job split (>= 1 Mi floats per job, <= 8 jobs), "
                          "same 36 B/element numerator",
                "host_cores_visible": os.cpu_count()}
-        if a.only == "all" and oracle.RefCompressor.available():
+        if a.only in ("all", "topk") and oracle.RefCompressor.available():
             ref = oracle.RefCompressor(2, 0.01)
             gh = grad[:BUCKET].cpu().numpy()
             ref.compress(gh, stable_id=1)

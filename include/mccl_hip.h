@@ -134,7 +134,7 @@ uint32_t mccl_hip_topk_k(uint64_t count, double ratio);
 /* TopKCompressor::max_compressed_size (TopKCompression.cpp:154-158). */
 uint64_t mccl_hip_topk_max_compressed_size(uint64_t nbytes, double ratio);
 /* Bytes of scratch mccl_hip_topk_compress needs for this shape. */
-uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems);
+uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, double ratio);
 
 /* TopKCompressor::compress (TopKCompression.cpp:38-120) for every bucket of a
  * gradient in one call.  grad and residual hold n_total fp32 elements, cut
@@ -151,6 +151,13 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
                            uint64_t bucket_elems, double ratio, void* wire,
                            uint64_t wire_stride, void* workspace, uint64_t workspace_bytes,
                            void* stream);
+
+/* Diagnostics, no counterpart in the reference: after a compress call on
+ * `stream` has been enqueued with this workspace and shape, waits for the
+ * stream and reports how many buckets were finished by the single-pass path
+ * (the others went through the exact fallback; results are identical). */
+int mccl_hip_topk_path_report(const void* workspace, uint64_t n_total, uint64_t bucket_elems, double ratio,
+                              uint32_t* host_single_pass_buckets, uint32_t* host_buckets, void* stream);
 
 /* TopKCompressor::decompress (TopKCompression.cpp:122-152): dense[0..count) is
  * zeroed, then dense[index] = value for every pair.  wire_bytes is the size

@@ -102,10 +102,12 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
     return v;
 }
 
-// Exclusive scan of one value per thread over a kBlock-thread block, in thread
-// order.  `smem` holds kBlock / kWave + 1 words.  Returns the exclusive prefix;
-// *total receives the block sum.  Ends with a barrier, so smem can be reused.
-__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* smem, uint32_t* total) {
+// Exclusive scan of one value per thread over a block of THREADS threads, in
+// thread order.  `smem` holds THREADS / kWave words.  Returns the exclusive
+// prefix; *total receives the block sum.  Ends with a barrier, so smem can be
+// reused.
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_exclusive_scan_n(uint32_t v, uint32_t* smem, uint32_t* total) {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     uint32_t inc = wave_inclusive_scan(v);
@@ -113,7 +115,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
     __syncthreads();
     uint32_t base = 0, sum = 0;
 #pragma unroll
-    for (int w = 0; w < kBlock / kWave; w++) {
+    for (int w = 0; w < THREADS / kWave; w++) {
         uint32_t s = smem[w];
         if (w < wave) base += s;
         sum += s;
@@ -121,6 +123,10 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
     __syncthreads();
     *total = sum;
     return base + inc - v;
+}
+
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* smem, uint32_t* total) {
+    return block_exclusive_scan_n<kBlock>(v, smem, total);
 }
 
 }  // namespace mcclhip

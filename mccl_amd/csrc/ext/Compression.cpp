@@ -49,7 +49,7 @@ size_t TopKCompressor::compress(const void* src, size_t nbytes, void* dst, size_
     }
     at::Tensor& residual = error_buffers_[stable_id];
 
-    const uint64_t ws_bytes = mccl_hip_topk_workspace_bytes(count, count);
+    const uint64_t ws_bytes = mccl_hip_topk_workspace_bytes(count, count, k_ratio_);
     if (!workspace_.defined() || static_cast<uint64_t>(workspace_.numel()) < ws_bytes) {
         workspace_ = at::empty({static_cast<int64_t>(ws_bytes)},
                                at::TensorOptions().dtype(at::kByte).device(at::kCUDA));

@@ -85,7 +85,7 @@ int mccl_hip_set_tuning(const char* key, int value) {
     } else if (!std::strcmp(key, "nontemporal")) {
         t.nontemporal = value ? 1 : 0;
     } else if (!std::strcmp(key, "topk_path")) {
-        if (value < 0 || value > 1) return MCCL_HIP_ERR_ARG;
+        if (value < 0 || value > 2) return MCCL_HIP_ERR_ARG;
         t.topk_path = value;
     } else {
         return MCCL_HIP_ERR_ARG;

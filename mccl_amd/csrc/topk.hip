@@ -7,47 +7,100 @@
 // threshold magnitude go to the lower index.
 //
 // For non-NaN floats, ordering by fabs() is ordering of the 31-bit pattern
-// `bits & 0x7FFFFFFF`, so selection is an exact radix select on that key:
-//   pass A      residual <- grad + residual, histogram of key[30:20]   (12 B/elem)
-//   pick        threshold bin, how many picks remain inside it
-//   refine x2   histograms of key[19:10] and key[9:0] among elements that match
-//               the prefix so far                                      (4 B/elem each)
-//   count       per 4096-element tile: #(key > T) and #(key == T)
-//   scan        exclusive prefix over tiles
-//   emit        ordered compaction: an element at index i lands at
-//               gt_before(i) + min(eq_before(i), need), ties accepted while
-//               eq_before(i) < need; residual[i] = 0 at every pick
+// `key = bits & 0x7FFFFFFF`, so selection is an exact radix select on that key.
 // All buckets of a gradient run in the same launches (blockIdx.y = bucket).
+//
+// FAST PATH (one pass over the gradient, 12 B/element of HBM traffic):
+//   sample     one block per bucket loads 12,288 evenly spread elements into
+//              LDS and radix-selects two of their keys: `lo`, which with 6 sigma
+//              of margin lies below the k-th largest key of the bucket, and
+//              `hi`, which with the same margin lies above it
+//   pass A     residual <- grad + residual in one streaming pass; elements with
+//              key >= lo ("candidates", about 1.7 k of them) are appended to
+//              per-bucket lists through per-wave LDS staging and counted in a
+//              2048-bin histogram that is linear in the key over [lo, hi)
+//   select1    finds the histogram bin that holds the k-th largest key and
+//              copies that bin's candidates (a handful) to a second list
+//   select2    one block per bucket: checks that the lists are complete and
+//              the threshold lies inside the window (else the bucket is handed
+//              to the exact fallback), finishes the radix select on the second
+//              list: exact threshold key T, how many keys equal to T are taken
+//              and - when not all of them are - the largest index still taken
+//   mark       sets one bit per pick in a bitmap of the bucket
+//   ecount     picks per 8192-element emission tile (popcount)
+//   emit       ordered compaction of the bitmap: index order comes for free;
+//              values are gathered from the residual, which is zeroed there
+// EXACT PATH (any input; also the per-bucket fallback of the fast path):
+//   [pass A]   residual <- grad + residual, histogram of key[30:20]
+//   refine x2  histograms of key[19:10], key[9:0] among prefix matches
+//   count      per 4096-element tile: #(key > T), #(key == T)
+//   emit       an element at index i lands at gt_before(i) + min(eq_before(i),
+//              need); ties are accepted while eq_before(i) < need
+//   Each kernel first derives the previous round's pick from the finished
+//   histogram (every block redundantly; the result is identical), so no
+//   separate pick launches are needed.
 #include "common.hip.h"
 #include "runtime.h"
+
+#include <vector>
 
 namespace mcclhip {
 
 namespace {
 
-constexpr int kTile = 4096;           // elements per compaction tile
-constexpr int kBins0 = 2048;          // key[30:20]
-constexpr int kBinsR = 1024;          // key[19:10], key[9:0]
+constexpr int kTile = 4096;    // exact path: elements per compaction tile
+constexpr int kBins0 = 2048;   // key[30:20]
+constexpr int kBinsR = 1024;   // key[19:10], key[9:0]
 constexpr int kHistWords = kBins0 + 2 * kBinsR;
-constexpr int kStateWords = 16;
+constexpr int kStateWords = 32;
+constexpr int kATile = 8192;   // fast path: elements per pass-A block
+constexpr int kETile = 8192;   // fast path: elements per emission block (256 bitmap words, one per thread)
+constexpr int kNSub = 64;      // fast path: candidate sub-lists per bucket
+constexpr int kStage = 512;    // fast path: staged candidates per wavefront
+constexpr int kSelThreads = 1024;
+constexpr uint64_t kFastMinBucket = 1u << 18;
+constexpr int kMarkTiles = 48;  // fast path: emission tiles one mark block can hold in LDS
+constexpr int kSample = 12288;  // fast path: sampled elements per bucket (12 per select thread)
 
 // per-bucket state words
-enum { S_PREFIX = 0, S_REMAIN = 1, S_GT_TOTAL = 2, S_EQ_TOTAL = 3 };
+enum {
+    S_P0 = 0, S_R0 = 1,   // key prefix / picks still to place after round 0
+    S_P1 = 2, S_R1 = 3,   // after round 1
+    S_T = 4, S_NEED = 5,  // exact threshold key, number of keys == T that are taken
+    S_LO_KEY = 6,         // fast path: candidates have key >= this
+    S_HI_KEY = 11,        // fast path: keys >= this fall into the top bin of the window histogram
+    S_SHIFT = 12,         // fast path: window bin = (key - lo) >> shift
+    S_OK = 7,             // fast path: 1 when select succeeded for this bucket
+    S_ISTAR = 8,          // fast path: ties are taken while index <= this
+    S_EXACT_HIST = 9,     // 1 when hist round 0 holds the full histogram
+    S_N2 = 10             // fast path: entries in list2
+};
 
 struct Geometry {
     uint64_t n_total;
     uint64_t bucket_elems;
     uint32_t nbuckets;
-    uint32_t tiles;   // tiles per (full) bucket
-    uint32_t k_full;  // k of a bucket with bucket_elems elements
-    uint32_t k_last;  // k of the last bucket
+    uint32_t tiles;    // exact-path tiles per (full) bucket
+    uint32_t k_full;   // k of a bucket with bucket_elems elements
+    uint32_t k_last;   // k of the last bucket
+    uint32_t etiles;   // emission tiles per bucket
+    uint32_t bwords;   // bitmap words per bucket (etiles * 256)
+    uint32_t lsub;     // capacity of one candidate sub-list (entries)
 };
 
 struct Workspace {
-    uint32_t* hist;     // [nbuckets][kHistWords]
-    uint32_t* state;    // [nbuckets][kStateWords]
-    uint32_t* tile_gt;  // [nbuckets][tiles]
-    uint32_t* tile_eq;  // [nbuckets][tiles]
+    // zeroed at the start of every exact-path call; the single-pass path zeroes what it uses itself
+    uint32_t* hist;         // [nbuckets][kHistWords]
+    uint32_t* hist_w;       // [nbuckets][kBins0]   candidates: window histogram, bin 2047 = above the window
+    uint32_t* state;        // [nbuckets][kStateWords]
+    uint32_t* sub_count;    // [nbuckets][kNSub]
+    uint32_t* etile_count;  // [nbuckets][etiles]
+    uint32_t* bitmap;       // [nbuckets][bwords]
+    // scratch, written before read
+    uint32_t* tile_gt;      // [nbuckets][tiles]
+    uint32_t* tile_eq;      // [nbuckets][tiles]
+    uint32_t* list;         // [nbuckets][kNSub][lsub][2]  (index, bits)
+    uint32_t* list2;        // [nbuckets][kNSub * lsub][2] candidates of the threshold bin
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -61,19 +114,64 @@ __device__ __forceinline__ uint32_t bucket_k(const Geometry& g, uint32_t b) {
 __device__ __forceinline__ uint32_t key_of(float v) { return f2u(v) & 0x7FFFFFFFu; }
 
 __global__ __launch_bounds__(kBlock) void k_zero_words(uint32_t* p, uint64_t n) {
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock)
-        p[i] = 0;
+    // n is a multiple of 4 and p is 16-byte aligned (see carve())
+    u4a* v = (u4a*)p;
+    const u4a z = {0u, 0u, 0u, 0u};
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n / 4; i += (uint64_t)gridDim.x * kBlock)
+        v[i] = z;
 }
 
 // Adds the block's LDS histogram into the bucket's global one (non-empty bins only).
+template <int THREADS>
 __device__ __forceinline__ void flush_hist(const uint32_t* lds, uint32_t* global, int bins) {
-    for (int i = threadIdx.x; i < bins; i += kBlock) {
+    for (int i = threadIdx.x; i < bins; i += THREADS) {
         uint32_t c = lds[i];
         if (c) atomicAdd(&global[i], c);
     }
 }
 
-// ---- pass A ---------------------------------------------------------------------
+// Scans a finished histogram from its top bin downwards and returns the bin in
+// which the running count reaches `remaining`, and through *left how many of
+// the remaining picks fall inside that bin.  Called by all THREADS threads of a
+// block with identical arguments; every thread receives the result.
+// `floor_bin`: bins below it count as empty.  Returns BINS when the histogram
+// holds fewer than `remaining` elements.
+template <int BINS, int THREADS>
+__device__ __forceinline__ uint32_t pick_bin(const uint32_t* h, uint32_t remaining, uint32_t floor_bin,
+                                             uint32_t* left, uint32_t* scratch /* THREADS/kWave + 2 words */) {
+    constexpr int PER = (BINS + THREADS - 1) / THREADS;
+    uint32_t c[PER];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int r = threadIdx.x * PER + j;  // reversed bin number
+        const int bin = BINS - 1 - r;
+        c[j] = (r < BINS && (uint32_t)bin >= floor_bin) ? h[bin] : 0u;
+        sum += c[j];
+    }
+    uint32_t total;
+    uint32_t above = block_exclusive_scan_n<THREADS>(sum, scratch, &total);
+    uint32_t* res = scratch + THREADS / kWave;
+    if (threadIdx.x == 0) { res[0] = BINS; res[1] = 0; }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        if (above < remaining && remaining <= above + c[j]) {
+            res[0] = BINS - 1 - (threadIdx.x * PER + j);
+            res[1] = remaining - above;
+        }
+        above += c[j];
+    }
+    __syncthreads();
+    const uint32_t bin = res[0];
+    *left = res[1];
+    __syncthreads();
+    return bin;
+}
+
+// ================================ exact path ======================================
+
+// residual <- grad + residual, histogram of key[30:20].
 __global__ __launch_bounds__(kBlock) void k_topk_pass_a(const float* __restrict__ grad, float* residual,
                                                         Geometry g, Workspace w) {
     __shared__ uint32_t lh[kBins0];
@@ -119,57 +217,64 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a(const float* __restrict_
         atomicAdd(&lh[key_of(adj) >> 20], 1u);
     }
     __syncthreads();
-    flush_hist(lh, w.hist + (uint64_t)b * kHistWords, kBins0);
+    flush_hist<kBlock>(lh, w.hist + (uint64_t)b * kHistWords, kBins0);
+    if (blockIdx.x == 0 && threadIdx.x == 0) w.state[(uint64_t)b * kStateWords + S_EXACT_HIST] = 1;
 }
 
-// ---- pick: one block per bucket ---------------------------------------------------
-// Finds the bin where the running count from the top bin downwards reaches the
-// number of picks still to place, narrows the key prefix to it, and keeps the
-// number of picks that fall inside it.
-template <int BINS>
-__global__ __launch_bounds__(kBlock) void k_topk_pick(Geometry g, Workspace w, int round) {
-    __shared__ uint32_t scan_smem[kBlock / kWave + 1];
-    constexpr int PER = BINS / kBlock;
-    const uint32_t b = blockIdx.x;
-    const int hist_off = round == 0 ? 0 : (round == 1 ? kBins0 : kBins0 + kBinsR);
-    const int shift = round == 0 ? 20 : (round == 1 ? 10 : 0);
-    const uint32_t* h = w.hist + (uint64_t)b * kHistWords + hist_off;
+// Derives (prefix, remaining) after `rounds_done` rounds for bucket b from the
+// finished histograms; block (0, b) also records them in the state.
+__device__ __forceinline__ void exact_prefix(const Geometry& g, const Workspace& w, uint32_t b, int rounds_done,
+                                             bool record, uint32_t* prefix, uint32_t* remaining,
+                                             uint32_t* scratch) {
+    const uint32_t* h = w.hist + (uint64_t)b * kHistWords;
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint32_t remaining = round == 0 ? bucket_k(g, b) : st[S_REMAIN];
-    const uint32_t prefix = round == 0 ? 0u : st[S_PREFIX];
-    // thread t owns bins descending from BINS-1 - t*PER
-    uint32_t c[PER];
-    uint32_t sum = 0;
-#pragma unroll
-    for (int j = 0; j < PER; j++) {
-        c[j] = h[BINS - 1 - (threadIdx.x * PER + j)];
-        sum += c[j];
+    uint32_t p = 0, r = bucket_k(g, b);
+    if (rounds_done >= 1) {
+        uint32_t left;
+        const uint32_t bin = pick_bin<kBins0, kBlock>(h, r, 0, &left, scratch);
+        p = bin << 20;
+        r = left;
+        if (record && rounds_done == 1 && threadIdx.x == 0) { st[S_P0] = p; st[S_R0] = r; }
     }
-    uint32_t total;
-    uint32_t above = block_exclusive_scan(sum, scan_smem, &total);
-#pragma unroll
-    for (int j = 0; j < PER; j++) {
-        if (above < remaining && remaining <= above + c[j]) {
-            const uint32_t bin = BINS - 1 - (threadIdx.x * PER + j);
-            st[S_PREFIX] = prefix | (bin << shift);
-            st[S_REMAIN] = remaining - above;
-        }
-        above += c[j];
+    if (rounds_done >= 2) {
+        uint32_t left;
+        const uint32_t bin = pick_bin<kBinsR, kBlock>(h + kBins0, r, 0, &left, scratch);
+        p |= bin << 10;
+        r = left;
+        if (record && rounds_done == 2 && threadIdx.x == 0) { st[S_P1] = p; st[S_R1] = r; }
     }
+    if (rounds_done >= 3) {
+        uint32_t left;
+        const uint32_t bin = pick_bin<kBinsR, kBlock>(h + kBins0 + kBinsR, r, 0, &left, scratch);
+        p |= bin;
+        r = left;
+        if (record && threadIdx.x == 0) { st[S_T] = p; st[S_NEED] = r; }
+    }
+    *prefix = p;
+    *remaining = r;
 }
 
-// ---- refine: histogram of the next key bits among prefix matches -------------------
+// round 0: full histogram of key[30:20] (only for buckets the fast path gave up on);
+// round 1 / 2: histogram of the next 10 key bits among elements matching the prefix.
 __global__ __launch_bounds__(kBlock) void k_topk_refine(const float* residual, Geometry g, Workspace w,
-                                                        int round) {
-    __shared__ uint32_t lh[kBinsR];
-    for (int i = threadIdx.x; i < kBinsR; i += kBlock) lh[i] = 0;
-    __syncthreads();
+                                                        int round, int only_failed) {
+    __shared__ uint32_t lh[kBins0];
+    __shared__ uint32_t scratch[kBlock / kWave + 2];
     const uint32_t b = blockIdx.y;
+    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    if (only_failed && st[S_OK]) return;
+    if (round == 0 && st[S_EXACT_HIST]) return;
+    const int bins = round == 0 ? kBins0 : kBinsR;
+    for (int i = threadIdx.x; i < bins; i += kBlock) lh[i] = 0;
+    uint32_t prefix = 0, remaining = 0;
+    if (round > 0) exact_prefix(g, w, b, round, blockIdx.x == 0, &prefix, &remaining, scratch);
+    __syncthreads();
     const uint64_t bn = bucket_count(g, b);
     const float* rp = residual + (uint64_t)b * g.bucket_elems;
-    const int shift = round == 1 ? 10 : 0;
-    const int hi_shift = shift + 10;
-    const uint32_t want = w.state[(uint64_t)b * kStateWords + S_PREFIX] >> hi_shift;
+    const int shift = round == 0 ? 20 : (round == 1 ? 10 : 0);
+    const int hi_shift = round == 0 ? 31 : shift + 10;
+    const uint32_t want = round == 0 ? 0u : prefix >> hi_shift;
+    const uint32_t mask = (uint32_t)bins - 1u;
     const uint64_t nvec = bn / 4;
     constexpr int U = 4;
     const uint64_t tile = (uint64_t)kBlock * U;
@@ -187,7 +292,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_refine(const float* residual, G
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const uint32_t key = v[u][q] & 0x7FFFFFFFu;
-                    if ((key >> hi_shift) == want) atomicAdd(&lh[(key >> shift) & (kBinsR - 1)], 1u);
+                    if ((key >> hi_shift) == want) atomicAdd(&lh[(key >> shift) & mask], 1u);
                 }
             }
         }
@@ -195,15 +300,14 @@ __global__ __launch_bounds__(kBlock) void k_topk_refine(const float* residual, G
     const uint64_t gtid = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (gtid < 4 && nvec * 4 + gtid < bn) {
         const uint32_t key = key_of(rp[nvec * 4 + gtid]);
-        if ((key >> hi_shift) == want) atomicAdd(&lh[(key >> shift) & (kBinsR - 1)], 1u);
+        if ((key >> hi_shift) == want) atomicAdd(&lh[(key >> shift) & mask], 1u);
     }
     __syncthreads();
-    flush_hist(lh, w.hist + (uint64_t)b * kHistWords + (round == 1 ? kBins0 : kBins0 + kBinsR), kBinsR);
+    const int off = round == 0 ? 0 : (round == 1 ? kBins0 : kBins0 + kBinsR);
+    flush_hist<kBlock>(lh, w.hist + (uint64_t)b * kHistWords + off, bins);
 }
 
-// ---- tiles ---------------------------------------------------------------------------
-// Loads the four keys of tile `t`, sub-tile `it`, lane slot; elements past the
-// bucket end read as "not selected" (valid = false).
+// Four consecutive elements of a tile; elements past the bucket end are invalid.
 struct Quad {
     uint32_t bits[4];
     bool valid[4];
@@ -227,127 +331,603 @@ __device__ __forceinline__ Quad load_quad(const float* rp, uint64_t bn, uint32_t
     return q;
 }
 
-__global__ __launch_bounds__(kBlock) void k_topk_count(const float* residual, Geometry g, Workspace w) {
-    __shared__ uint32_t red[kBlock / kWave + 1];
-    const uint32_t b = blockIdx.y, t = blockIdx.x;
+__global__ __launch_bounds__(kBlock) void k_topk_count(const float* residual, Geometry g, Workspace w,
+                                                       int only_failed) {
+    __shared__ uint32_t scratch[kBlock / kWave + 2];
+    const uint32_t b = blockIdx.y;
+    if (only_failed && w.state[(uint64_t)b * kStateWords + S_OK]) return;
     const uint64_t bn = bucket_count(g, b);
-    if ((uint64_t)t * kTile >= bn) {
-        if (threadIdx.x == 0) {
-            w.tile_gt[(uint64_t)b * g.tiles + t] = 0;
-            w.tile_eq[(uint64_t)b * g.tiles + t] = 0;
-        }
-        return;
-    }
     const float* rp = residual + (uint64_t)b * g.bucket_elems;
-    const uint32_t T = w.state[(uint64_t)b * kStateWords + S_PREFIX];
-    uint32_t packed = 0;  // gt in the low half, eq in the high half (each <= 4096)
+    uint32_t T, need;
+    exact_prefix(g, w, b, 3, blockIdx.x == 0, &T, &need, scratch);
+    for (uint32_t t = blockIdx.x; t < g.tiles; t += gridDim.x) {
+        uint32_t packed = 0;  // gt in the low half, eq in the high half (each <= 4096)
+        if ((uint64_t)t * kTile < bn) {
 #pragma unroll
-    for (int it = 0; it < kTile / (kBlock * 4); it++) {
-        Quad q = load_quad(rp, bn, t, it);
+            for (int it = 0; it < kTile / (kBlock * 4); it++) {
+                Quad q = load_quad(rp, bn, t, it);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t key = q.bits[j] & 0x7FFFFFFFu;
-            if (q.valid[j]) packed += (key > T ? 1u : 0u) + (key == T ? 0x10000u : 0u);
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t key = q.bits[j] & 0x7FFFFFFFu;
+                    if (q.valid[j]) packed += (key > T ? 1u : 0u) + (key == T ? 0x10000u : 0u);
+                }
+            }
         }
-    }
-    uint32_t total;
-    block_exclusive_scan(packed, red, &total);
-    if (threadIdx.x == 0) {
-        w.tile_gt[(uint64_t)b * g.tiles + t] = total & 0xFFFFu;
-        w.tile_eq[(uint64_t)b * g.tiles + t] = total >> 16;
-    }
-}
-
-// One block per bucket: in-place exclusive scan of the tile counts.
-__global__ __launch_bounds__(kBlock) void k_topk_scan(Geometry g, Workspace w) {
-    __shared__ uint32_t smem[kBlock / kWave + 1];
-    const uint32_t b = blockIdx.x;
-    uint32_t* gt = w.tile_gt + (uint64_t)b * g.tiles;
-    uint32_t* eq = w.tile_eq + (uint64_t)b * g.tiles;
-    uint32_t carry_gt = 0, carry_eq = 0;
-    for (uint32_t base = 0; base < g.tiles; base += kBlock) {
-        const uint32_t i = base + threadIdx.x;
-        const uint32_t a = i < g.tiles ? gt[i] : 0u;
-        const uint32_t e = i < g.tiles ? eq[i] : 0u;
-        uint32_t ta, te;
-        const uint32_t xa = block_exclusive_scan(a, smem, &ta);
-        const uint32_t xe = block_exclusive_scan(e, smem, &te);
-        if (i < g.tiles) {
-            gt[i] = carry_gt + xa;
-            eq[i] = carry_eq + xe;
+        uint32_t total;
+        block_exclusive_scan(packed, scratch, &total);
+        if (threadIdx.x == 0) {
+            w.tile_gt[(uint64_t)b * g.tiles + t] = total & 0xFFFFu;
+            w.tile_eq[(uint64_t)b * g.tiles + t] = total >> 16;
         }
-        carry_gt += ta;
-        carry_eq += te;
-    }
-    if (threadIdx.x == 0) {
-        w.state[(uint64_t)b * kStateWords + S_GT_TOTAL] = carry_gt;
-        w.state[(uint64_t)b * kStateWords + S_EQ_TOTAL] = carry_eq;
     }
 }
 
 __global__ __launch_bounds__(kBlock) void k_topk_emit(float* residual, Geometry g, Workspace w,
-                                                      uint8_t* wire, uint64_t wire_stride) {
-    __shared__ uint32_t smem[kBlock / kWave + 1];
-    const uint32_t b = blockIdx.y, t = blockIdx.x;
+                                                      uint8_t* wire, uint64_t wire_stride, int only_failed) {
+    __shared__ uint32_t smem[kBlock / kWave + 2];
+    const uint32_t b = blockIdx.y;
+    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    if (only_failed && st[S_OK]) return;
     const uint64_t bn = bucket_count(g, b);
     uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
-    if (t == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
-    if ((uint64_t)t * kTile >= bn) return;
+    if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
     float* rp = residual + (uint64_t)b * g.bucket_elems;
-    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint32_t T = st[S_PREFIX];
-    const uint32_t need = st[S_REMAIN];
-    uint32_t gt_run = w.tile_gt[(uint64_t)b * g.tiles + t];
-    uint32_t eq_run = w.tile_eq[(uint64_t)b * g.tiles + t];
+    const uint32_t T = st[S_T];
+    const uint32_t need = st[S_NEED];
+    const uint32_t* tgt = w.tile_gt + (uint64_t)b * g.tiles;
+    const uint32_t* teq = w.tile_eq + (uint64_t)b * g.tiles;
+    for (uint32_t t = blockIdx.x; t < g.tiles; t += gridDim.x) {
+        if ((uint64_t)t * kTile >= bn) break;
+        // picks before this tile: sum of the counts of all earlier tiles
+        uint32_t sg = 0, se = 0;
+        for (uint32_t i = threadIdx.x; i < t; i += kBlock) { sg += tgt[i]; se += teq[i]; }
+        uint32_t gt_run, eq_run;
+        block_exclusive_scan(sg, smem, &gt_run);
+        block_exclusive_scan(se, smem, &eq_run);
 #pragma unroll 1
-    for (int it = 0; it < kTile / (kBlock * 4); it++) {
-        Quad q = load_quad(rp, bn, t, it);
-        uint32_t packed = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t key = q.bits[j] & 0x7FFFFFFFu;
-            if (q.valid[j]) packed += (key > T ? 1u : 0u) + (key == T ? 0x10000u : 0u);
-        }
-        uint32_t total;
-        const uint32_t ex = block_exclusive_scan(packed, smem, &total);
-        uint32_t gt_b = gt_run + (ex & 0xFFFFu);
-        uint32_t eq_b = eq_run + (ex >> 16);
-        if (packed) {
+        for (int it = 0; it < kTile / (kBlock * 4); it++) {
+            Quad q = load_quad(rp, bn, t, it);
+            uint32_t packed = 0;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t key = q.bits[j] & 0x7FFFFFFFu;
-                const bool is_gt = q.valid[j] && key > T;
-                const bool is_eq = q.valid[j] && key == T;
-                if (is_gt || (is_eq && eq_b < need)) {
-                    const uint32_t pos = gt_b + (eq_b < need ? eq_b : need);
-                    out[1 + 2 * (uint64_t)pos] = (uint32_t)(q.e + j);
-                    out[2 + 2 * (uint64_t)pos] = q.bits[j];
-                    rp[q.e + j] = 0.0f;
-                }
-                gt_b += is_gt ? 1u : 0u;
-                eq_b += is_eq ? 1u : 0u;
+                if (q.valid[j]) packed += (key > T ? 1u : 0u) + (key == T ? 0x10000u : 0u);
             }
+            uint32_t total;
+            const uint32_t ex = block_exclusive_scan(packed, smem, &total);
+            uint32_t gt_b = gt_run + (ex & 0xFFFFu);
+            uint32_t eq_b = eq_run + (ex >> 16);
+            if (packed) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t key = q.bits[j] & 0x7FFFFFFFu;
+                    const bool is_gt = q.valid[j] && key > T;
+                    const bool is_eq = q.valid[j] && key == T;
+                    if (is_gt || (is_eq && eq_b < need)) {
+                        const uint32_t pos = gt_b + (eq_b < need ? eq_b : need);
+                        out[1 + 2 * (uint64_t)pos] = (uint32_t)(q.e + j);
+                        out[2 + 2 * (uint64_t)pos] = q.bits[j];
+                        rp[q.e + j] = 0.0f;
+                    }
+                    gt_b += is_gt ? 1u : 0u;
+                    eq_b += is_eq ? 1u : 0u;
+                }
+            }
+            gt_run += total & 0xFFFFu;
+            eq_run += total >> 16;
+        }
+    }
+}
+
+// ================================= fast path ======================================
+
+// Window bin of a candidate key: linear in the key over [lo, hi), everything
+// at or above hi in bin kBins0 - 1.
+__device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32_t hi, uint32_t shift) {
+    return key >= hi ? (uint32_t)(kBins0 - 1) : (key - lo) >> shift;
+}
+
+// One block per bucket.  Loads kSample evenly spread elements of grad + residual
+// into LDS and radix-selects (11 + 10 + 10 key bits, both ranks in the same
+// sweeps) the keys of sample ranks
+//     r_hi = ks - 6 sqrt(ks) - 16   and   r_lo = ks + 6 sqrt(ks) + 16,
+// ks = k * S / n being the expected number of sampled elements among the top k.
+__global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __restrict__ grad,
+                                                             const float* __restrict__ residual, Geometry g,
+                                                             Workspace w) {
+    __shared__ uint32_t keys[kSample];
+    __shared__ uint32_t lh[2][kBinsR];
+    __shared__ uint32_t scratch[kSelThreads / kWave + 2];
+    const uint32_t b = blockIdx.x;
+    // this bucket's accumulators for the kernels that follow start at zero
+    for (int i = threadIdx.x; i < kBins0; i += kSelThreads) w.hist_w[(uint64_t)b * kBins0 + i] = 0;
+    if (threadIdx.x < kNSub) w.sub_count[(uint64_t)b * kNSub + threadIdx.x] = 0;
+    if (threadIdx.x < kStateWords) w.state[(uint64_t)b * kStateWords + threadIdx.x] = 0;
+    const uint64_t bn = bucket_count(g, b);
+    const float* gp = grad + (uint64_t)b * g.bucket_elems;
+    const float* rp = residual + (uint64_t)b * g.bucket_elems;
+    const uint64_t nvec = bn / 4;
+    constexpr int SV = kSample / 4;  // sampled vectors
+    const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)nvec : (uint32_t)SV;
+    const uint64_t stride = nsv ? nvec / nsv : 1;
+    u4a gv[SV / kSelThreads], rv[SV / kSelThreads];
+#pragma unroll
+    for (int j = 0; j < SV / kSelThreads; j++) {
+        const uint32_t i = (uint32_t)j * kSelThreads + threadIdx.x;
+        const uint64_t v = (uint64_t)(i < nsv ? i : 0) * stride;
+        gv[j] = nsv ? *(const u4u4*)(gp + v * 4) : u4a{0u, 0u, 0u, 0u};
+        rv[j] = nsv ? *(const u4u4*)(rp + v * 4) : u4a{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int j = 0; j < SV / kSelThreads; j++) {
+        const uint32_t i = (uint32_t)j * kSelThreads + threadIdx.x;
+#pragma unroll
+        for (int q = 0; q < 4; q++) keys[4 * i + q] = i < nsv ? key_of(u2f(gv[j][q]) + u2f(rv[j][q])) : 0u;
+    }
+    const uint32_t S = nsv * 4;
+    const float ks = (float)bucket_k(g, b) * (float)S / (float)bn;
+    const float margin = 6.0f * sqrtf(ks) + 16.0f;
+    uint32_t rank[2];
+    rank[0] = ks - margin >= 1.0f ? (uint32_t)(ks - margin) : 0u;  // 0: no upper end
+    rank[1] = (uint32_t)(ks + margin) + 1u;                       // > S: no lower end
+    uint32_t prefix[2] = {0u, 0u}, want[2] = {rank[0], rank[1]};
+    const bool active[2] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S};
+    const int shifts[3] = {20, 10, 0};
+    __syncthreads();
+    for (int r = 0; r < 3; r++) {
+        // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves both ranks
+        uint32_t* h0 = &lh[0][0];
+        for (int i = threadIdx.x; i < 2 * kBinsR; i += kSelThreads) h0[i] = 0;
+        __syncthreads();
+        const int shift = shifts[r];
+        for (uint32_t i = threadIdx.x; i < S; i += kSelThreads) {
+            const uint32_t key = keys[i];
+            if (r == 0) {
+                atomicAdd(&h0[key >> 20], 1u);
+            } else {
+                const int hs = shift + 10;
+#pragma unroll
+                for (int z = 0; z < 2; z++)
+                    if (active[z] && (key >> hs) == (prefix[z] >> hs)) atomicAdd(&lh[z][(key >> shift) & (kBinsR - 1)], 1u);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int z = 0; z < 2; z++) {
+            if (!active[z]) continue;
+            uint32_t left, bin;
+            if (r == 0) bin = pick_bin<kBins0, kSelThreads>(h0, want[z], 0, &left, scratch);
+            else bin = pick_bin<kBinsR, kSelThreads>(lh[z], want[z], 0, &left, scratch);
+            prefix[z] |= bin << shift;
+            want[z] = left;
+        }
+    }
+    if (threadIdx.x == 0) {
+        const uint32_t lo = active[1] ? prefix[1] : 0u;
+        uint32_t hi = active[0] ? prefix[0] : 0x7FFFFFFFu;
+        if (hi < lo) hi = lo;
+        uint32_t shift = 0;
+        while (((hi - lo) >> shift) >= (uint32_t)(kBins0 - 1)) shift++;
+        uint32_t* st = w.state + (uint64_t)b * kStateWords;
+        st[S_LO_KEY] = lo;
+        st[S_HI_KEY] = hi;
+        st[S_SHIFT] = shift;
+    }
+}
+
+// residual <- grad + residual; candidates (key >= lo) are counted in the window
+// histogram and appended to the bucket's sub-list (tile number mod kNSub).
+// One 8192-element tile per block, tiles in address order.
+__global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __restrict__ grad, float* residual,
+                                                             Geometry g, Workspace w) {
+    __shared__ uint32_t lh[kBins0];
+    __shared__ uint32_t stage[kBlock / kWave][kStage][2];
+    const uint32_t b = blockIdx.y, t = blockIdx.x;
+    const uint64_t bn = bucket_count(g, b);
+    const uint64_t e0 = (uint64_t)t * kATile;
+    if (e0 >= bn) return;
+    for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
+    __syncthreads();
+    const float* gp = grad + (uint64_t)b * g.bucket_elems;
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    const uint32_t lo_key = w.state[(uint64_t)b * kStateWords + S_LO_KEY];
+    const uint32_t hi_key = w.state[(uint64_t)b * kStateWords + S_HI_KEY];
+    const uint32_t wshift = w.state[(uint64_t)b * kStateWords + S_SHIFT];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const uint32_t sub = t % kNSub;
+    uint32_t* sub_cnt = w.sub_count + (uint64_t)b * kNSub + sub;
+    uint32_t* sub_list = w.list + (((uint64_t)b * kNSub + sub) * g.lsub) * 2;
+    uint32_t staged = 0;  // wave-uniform
+
+    auto flush_stage = [&]() {
+        uint32_t base = 0;
+        if (lane == 0) base = atomicAdd(sub_cnt, staged);
+        base = __shfl(base, 0, kWave);
+        for (uint32_t i = lane; i < staged; i += kWave) {
+            const uint32_t pos = base + i;
+            if (pos < g.lsub) {
+                sub_list[2 * (uint64_t)pos] = stage[wave][i][0];
+                sub_list[2 * (uint64_t)pos + 1] = stage[wave][i][1];
+            }
+        }
+        staged = 0;
+    };
+
+    constexpr int U = 4;
+    const uint64_t tile_end = (e0 + kATile) < bn ? (e0 + kATile) : bn;
+    const uint64_t nfull = (tile_end - e0) / 4;  // full vectors in this tile
+#pragma unroll 1
+    for (int round = 0; round < kATile / (kBlock * 4 * U); round++) {
+        u4a gv[U], rv[U];
+        uint64_t vi[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            vi[u] = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
+            if (vi[u] < nfull) {
+                gv[u] = __builtin_nontemporal_load((const u4u4*)(gp + e0 + vi[u] * 4));
+                rv[u] = __builtin_nontemporal_load((const u4u4*)(rp + e0 + vi[u] * 4));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            u4a a = {0u, 0u, 0u, 0u};
+            bool cand[4] = {false, false, false, false};
+            const bool live = vi[u] < nfull;
+            if (live) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float adj = u2f(gv[u][q]) + u2f(rv[u][q]);
+                    a[q] = f2u(adj);
+                    cand[q] = key_of(adj) >= lo_key;
+                }
+                __builtin_nontemporal_store(a, (u4u4*)(rp + e0 + vi[u] * 4));
+            }
+            const bool any = cand[0] | cand[1] | cand[2] | cand[3];
+            if (__ballot(any)) {  // wave-uniform
+                if (staged + 4 * kWave > kStage) flush_stage();
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint64_t m = __ballot(cand[q]);
+                    if (cand[q]) {
+                        const uint32_t pos = staged + __popcll(m & ((1ull << lane) - 1ull));
+                        stage[wave][pos][0] = (uint32_t)(e0 + vi[u] * 4 + q);
+                        stage[wave][pos][1] = a[q];
+                        atomicAdd(&lh[window_bin(a[q] & 0x7FFFFFFFu, lo_key, hi_key, wshift)], 1u);
+                    }
+                    staged += (uint32_t)__popcll(m);
+                }
+            }
+        }
+    }
+    // the bucket's last partial vector (bucket length not a multiple of 4)
+    if (tile_end == bn && (bn & 3) && wave == 0) {
+        const uint64_t i = e0 + nfull * 4 + lane;
+        bool c = false;
+        uint32_t bitsv = 0;
+        if (lane < 4 && i < bn) {
+            const float adj = gp[i] + rp[i];
+            rp[i] = adj;
+            bitsv = f2u(adj);
+            c = key_of(adj) >= lo_key;
+        }
+        const uint64_t m = __ballot(c);
+        if (m) {
+            if (staged + kWave > kStage) flush_stage();
+            if (c) {
+                const uint32_t pos = staged + __popcll(m & ((1ull << lane) - 1ull));
+                stage[wave][pos][0] = (uint32_t)i;
+                stage[wave][pos][1] = bitsv;
+                atomicAdd(&lh[window_bin(bitsv & 0x7FFFFFFFu, lo_key, hi_key, wshift)], 1u);
+            }
+            staged += (uint32_t)__popcll(m);
+        }
+    }
+    if (staged) flush_stage();
+    __syncthreads();
+    flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kBins0, kBins0);
+}
+
+// A block's view of up to 8 * kBlock consecutive (index, bits) entries: all
+// loads are issued before the first use.
+struct EntryChunk {
+    uint32_t idx[8], bits[8];
+    bool valid[8];
+};
+__device__ __forceinline__ EntryChunk load_entries(const uint32_t* l, uint32_t base, uint32_t cnt) {
+    EntryChunk c;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t i = base + (uint32_t)j * kBlock + threadIdx.x;
+        c.valid[j] = i < cnt;
+        const uint32_t ii = c.valid[j] ? i : 0u;
+        c.idx[j] = l[2 * (uint64_t)ii];
+        c.bits[j] = l[2 * (uint64_t)ii + 1];
+    }
+    return c;
+}
+
+// select, step 1: one block per candidate sub-list.  Finds the window bin that
+// holds the k-th largest key (every block gets the same answer) and copies that
+// bin's candidates to list2 (order irrelevant): the rest of the selection only
+// touches those.
+__global__ __launch_bounds__(kBlock) void k_topk_select1(Geometry g, Workspace w) {
+    __shared__ uint32_t scratch[kBlock / kWave + 2];
+    __shared__ uint32_t gbase;
+    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
+    uint32_t need;
+    const uint32_t jstar = pick_bin<kBins0, kBlock>(w.hist_w + (uint64_t)b * kBins0, bucket_k(g, b), 0, &need, scratch);
+    if (s == 0 && threadIdx.x == 0) { st[S_P0] = jstar; st[S_R0] = need; }
+    // fewer than k candidates, or the threshold lies above the window: fallback
+    if (jstar >= (uint32_t)(kBins0 - 1)) return;
+    uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
+    if (cnt > g.lsub) cnt = g.lsub;
+    const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
+    uint32_t* l2 = w.list2 + ((uint64_t)b * kNSub * g.lsub) * 2;
+    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
+        const EntryChunk c = load_entries(l, base, cnt);
+        uint32_t mine = 0;
+        bool hit[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
+            hit[j] = c.valid[j] && window_bin(key, lo, hi, shift) == jstar;
+            mine += hit[j] ? 1u : 0u;
+        }
+        uint32_t total;
+        uint32_t pos = block_exclusive_scan(mine, scratch, &total);
+        if (total) {  // uniform
+            if (threadIdx.x == 0) gbase = atomicAdd(st + S_N2, total);
+            __syncthreads();
+            pos += gbase;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (hit[j]) {
+                    l2[2 * (uint64_t)pos] = c.idx[j];
+                    l2[2 * (uint64_t)pos + 1] = c.bits[j] & 0x7FFFFFFFu;
+                    pos++;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// Whole exact selection of one bucket by one block: the fallback for buckets
+// whose candidate lists turned out incomplete.  Slow (one block streams the
+// bucket five times) but costs no extra launch: select2 calls it in place.
+// lh: kBins0 words, scratch: kSelThreads / kWave + 2 words of LDS.
+__device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uint8_t* wire, uint64_t wire_stride,
+                             uint32_t* lh, uint32_t* scratch) {
+    const uint64_t bn = bucket_count(g, b);
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    uint32_t prefix = 0, remaining = bucket_k(g, b);
+    for (int round = 0; round < 3; round++) {
+        const int bins = round == 0 ? kBins0 : kBinsR;
+        const int shift = round == 0 ? 20 : (round == 1 ? 10 : 0);
+        const int hi_shift = round == 0 ? 31 : shift + 10;
+        for (int i = threadIdx.x; i < kBins0; i += kSelThreads) lh[i] = 0;
+        __syncthreads();
+        for (uint64_t i = threadIdx.x; i < bn; i += kSelThreads) {
+            const uint32_t key = key_of(rp[i]);
+            if ((key >> hi_shift) == (prefix >> hi_shift)) atomicAdd(&lh[(key >> shift) & (bins - 1)], 1u);
+        }
+        __syncthreads();
+        uint32_t left, bin;
+        if (round == 0) bin = pick_bin<kBins0, kSelThreads>(lh, remaining, 0, &left, scratch);
+        else bin = pick_bin<kBinsR, kSelThreads>(lh, remaining, 0, &left, scratch);
+        prefix |= bin << shift;
+        remaining = left;
+    }
+    const uint32_t T = prefix, need = remaining;
+    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
+    if (threadIdx.x == 0) out[0] = bucket_k(g, b);
+    uint32_t gt_run = 0, eq_run = 0;
+    for (uint64_t base = 0; base < bn; base += kSelThreads) {
+        const uint64_t i = base + threadIdx.x;
+        const uint32_t bitsv = i < bn ? f2u(rp[i]) : 0u;
+        const uint32_t key = bitsv & 0x7FFFFFFFu;
+        const bool is_gt = i < bn && key > T;
+        const bool is_eq = i < bn && key == T;
+        uint32_t total;
+        const uint32_t ex = block_exclusive_scan_n<kSelThreads>((is_gt ? 1u : 0u) + (is_eq ? 0x10000u : 0u), scratch,
+                                                                &total);
+        const uint32_t gt_b = gt_run + (ex & 0xFFFFu), eq_b = eq_run + (ex >> 16);
+        if (is_gt || (is_eq && eq_b < need)) {
+            const uint32_t pos = gt_b + (eq_b < need ? eq_b : need);
+            out[1 + 2 * (uint64_t)pos] = (uint32_t)i;
+            out[2 + 2 * (uint64_t)pos] = bitsv;
+            rp[i] = 0.0f;
         }
         gt_run += total & 0xFFFFu;
         eq_run += total >> 16;
     }
 }
 
+// select, step 2: one block per bucket.  Validates the candidate lists, finishes
+// the radix select on list2 (keys of one window bin: 21 bits at most remain)
+// and resolves ties by index.
+__global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, Geometry g, Workspace w,
+                                                              uint8_t* wire, uint64_t wire_stride) {
+    __shared__ uint32_t lh[kBins0];
+    __shared__ uint32_t scratch[kSelThreads / kWave + 2];
+    const uint32_t b = blockIdx.x;
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    const uint32_t jstar = st[S_P0];
+    uint32_t want = st[S_R0];
+    uint32_t over = 0;
+    if (threadIdx.x < kNSub) over = w.sub_count[(uint64_t)b * kNSub + threadIdx.x] > g.lsub ? 1u : 0u;
+    uint32_t any_over;
+    block_exclusive_scan_n<kSelThreads>(over, scratch, &any_over);
+    if (any_over || jstar >= (uint32_t)(kBins0 - 1)) {
+        // incomplete candidate lists or threshold outside the window (rare): this block
+        // runs the whole exact selection of the bucket; S_OK stays 0, so mark and emit skip it
+        bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
+        return;
+    }
+
+    const uint32_t* l2 = w.list2 + ((uint64_t)b * kNSub * g.lsub) * 2;
+    const uint32_t count2 = st[S_N2];
+    const uint32_t bin_lo = st[S_LO_KEY] + (jstar << st[S_SHIFT]);  // smallest key of the bin
+    uint32_t vprefix = 0;  // key - bin_lo: up to 21 bits, selected as 1 + 10 + 10
+    for (int r = 0; r < 3; r++) {
+        const int shift = 20 - 10 * r;
+        const int hs = shift + 10;
+        for (int i = threadIdx.x; i < kBinsR; i += kSelThreads) lh[i] = 0;
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < count2; i += kSelThreads) {
+            const uint32_t v = l2[2 * (uint64_t)i + 1] - bin_lo;
+            if ((v >> hs) == (vprefix >> hs)) atomicAdd(&lh[(v >> shift) & (kBinsR - 1)], 1u);
+        }
+        __syncthreads();
+        uint32_t left;
+        const uint32_t bin = pick_bin<kBinsR, kSelThreads>(lh, want, 0, &left, scratch);
+        vprefix |= bin << shift;
+        want = left;
+    }
+    const uint32_t T = bin_lo + vprefix;
+    const uint32_t need2 = want;
+    const uint32_t ties = lh[vprefix & (kBinsR - 1)];
+    __syncthreads();
+
+    // ties: when only some keys equal to T are taken, they are the `need2` lowest
+    // indices: radix-select the need2-th smallest index (11 + 11 + 10 bits)
+    uint32_t istar = 0xFFFFFFFFu;
+    if (ties != need2) {
+        uint32_t iwant = need2, iprefix = 0;
+        const int shifts[3] = {21, 10, 0};
+        const int widths[3] = {11, 11, 10};
+        for (int r = 0; r < 3; r++) {
+            const int bins = 1 << widths[r];
+            for (int i = threadIdx.x; i < kBins0; i += kSelThreads) lh[i] = 0;
+            __syncthreads();
+            const int hs = shifts[r] + widths[r];
+            for (uint32_t i = threadIdx.x; i < count2; i += kSelThreads) {
+                const uint32_t idx = l2[2 * (uint64_t)i], key = l2[2 * (uint64_t)i + 1];
+                const bool match = hs >= 32 ? true : ((idx >> hs) == (iprefix >> hs));
+                // bins stored reversed, so that pick_bin's top-down scan runs over ascending indices
+                if (key == T && match) atomicAdd(&lh[(bins - 1) - ((idx >> shifts[r]) & (bins - 1))], 1u);
+            }
+            __syncthreads();
+            uint32_t left, rb;
+            if (bins == kBins0) rb = pick_bin<kBins0, kSelThreads>(lh, iwant, 0, &left, scratch);
+            else rb = pick_bin<kBinsR, kSelThreads>(lh, iwant, 0, &left, scratch);
+            iprefix |= ((uint32_t)(bins - 1) - rb) << shifts[r];
+            iwant = left;
+        }
+        istar = iprefix;
+    }
+    if (threadIdx.x == 0) {
+        st[S_T] = T;
+        st[S_NEED] = need2;
+        st[S_ISTAR] = istar;
+        st[S_OK] = 1;
+    }
+}
+
+// One block per candidate sub-list.  A sub-list holds the candidates of the
+// pass-A tiles t = s, s + kNSub, ...; an emission tile is the same 8192 elements,
+// so this block owns those tiles' bitmap words outright: it builds them in LDS,
+// stores them whole (no atomics, no pre-zeroed bitmap) and counts their picks.
+__global__ __launch_bounds__(kBlock) void k_topk_mark(Geometry g, Workspace w) {
+    __shared__ uint32_t bm[kMarkTiles * (kETile / 32)];
+    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    if (!st[S_OK]) return;
+    const uint32_t T = st[S_T], istar = st[S_ISTAR];
+    const uint32_t ntiles = s < g.etiles ? (g.etiles - s + kNSub - 1) / kNSub : 0u;  // tiles of this sub-list
+    for (uint32_t i = threadIdx.x; i < ntiles * (kETile / 32); i += kBlock) bm[i] = 0;
+    __syncthreads();
+    uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
+    if (cnt > g.lsub) cnt = g.lsub;
+    const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
+    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
+        const EntryChunk c = load_entries(l, base, cnt);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
+            if (c.valid[j] && (key > T || (key == T && c.idx[j] <= istar))) {
+                const uint32_t tile = c.idx[j] / kETile;            // == s (mod kNSub)
+                const uint32_t word = (tile / kNSub) * (kETile / 32) + ((c.idx[j] % kETile) >> 5);
+                atomicOr(&bm[word], 1u << (c.idx[j] & 31));
+            }
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1);
+    for (uint32_t j = threadIdx.x / kWave; j < ntiles; j += kBlock / kWave) {  // one wavefront per tile
+        const uint32_t tile = s + j * kNSub;
+        const u4a v = ((const u4a*)(bm + j * (kETile / 32)))[lane];
+        ((u4a*)(w.bitmap + (uint64_t)b * g.bwords + (uint64_t)tile * (kETile / 32)))[lane] = v;
+        uint32_t c = __popc(v[0]) + __popc(v[1]) + __popc(v[2]) + __popc(v[3]);
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) c += __shfl_xor(c, d, kWave);
+        if (lane == 0) w.etile_count[(uint64_t)b * g.etiles + tile] = c;
+    }
+}
+
+// Ordered compaction of the bitmap: 256 words per block, one per thread.
+__global__ __launch_bounds__(kBlock) void k_topk_emit_fast(float* residual, Geometry g, Workspace w,
+                                                           uint8_t* wire, uint64_t wire_stride) {
+    __shared__ uint32_t smem[kBlock / kWave + 2];
+    const uint32_t b = blockIdx.y, t = blockIdx.x;
+    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    if (!st[S_OK]) return;
+    const uint64_t bn = bucket_count(g, b);
+    if ((uint64_t)t * kETile >= bn) return;
+    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
+    if (t == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    const uint32_t* ec = w.etile_count + (uint64_t)b * g.etiles;
+    uint32_t before = 0;
+    for (uint32_t i = threadIdx.x; i < t; i += kBlock) before += ec[i];
+    uint32_t base;
+    block_exclusive_scan(before, smem, &base);
+    uint32_t m = w.bitmap[(uint64_t)b * g.bwords + (uint64_t)t * (kETile / 32) + threadIdx.x];
+    uint32_t total;
+    uint32_t pos = base + block_exclusive_scan((uint32_t)__popc(m), smem, &total);
+    while (m) {
+        const int bit = __ffs(m) - 1;
+        m &= m - 1;
+        const uint32_t idx = t * (uint32_t)kETile + threadIdx.x * 32u + (uint32_t)bit;
+        out[1 + 2 * (uint64_t)pos] = idx;
+        out[2 + 2 * (uint64_t)pos] = f2u(rp[idx]);
+        rp[idx] = 0.0f;
+        pos++;
+    }
+}
+
+// ================================ host side =======================================
+
+uint64_t align4(uint64_t words) { return (words + 3) & ~uint64_t(3); }
+
+uint64_t zeroed_words(const Geometry& g) {
+    return align4((uint64_t)g.nbuckets * kHistWords) + align4((uint64_t)g.nbuckets * kBins0) +
+           align4((uint64_t)g.nbuckets * kStateWords) + align4((uint64_t)g.nbuckets * kNSub);
+}
+
+uint64_t workspace_words(const Geometry& g) {
+    return zeroed_words(g) + align4((uint64_t)g.nbuckets * g.etiles) + align4((uint64_t)g.nbuckets * g.bwords) +
+           2 * align4((uint64_t)g.nbuckets * g.tiles) +
+           2 * align4((uint64_t)g.nbuckets * kNSub * g.lsub * 2);
+}
+
 Workspace carve(void* base, const Geometry& g) {
     Workspace w;
     uint32_t* p = (uint32_t*)base;
-    w.hist = p;
-    p += (uint64_t)g.nbuckets * kHistWords;
-    w.state = p;
-    p += (uint64_t)g.nbuckets * kStateWords;
-    w.tile_gt = p;
-    p += (uint64_t)g.nbuckets * g.tiles;
-    w.tile_eq = p;
+    w.hist = p;        p += align4((uint64_t)g.nbuckets * kHistWords);
+    w.hist_w = p;      p += align4((uint64_t)g.nbuckets * kBins0);
+    w.state = p;       p += align4((uint64_t)g.nbuckets * kStateWords);
+    w.sub_count = p;   p += align4((uint64_t)g.nbuckets * kNSub);
+    w.etile_count = p; p += align4((uint64_t)g.nbuckets * g.etiles);
+    w.bitmap = p;      p += align4((uint64_t)g.nbuckets * g.bwords);
+    w.tile_gt = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
+    w.tile_eq = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
+    w.list = p;        p += align4((uint64_t)g.nbuckets * kNSub * g.lsub * 2);
+    w.list2 = p;
     return w;
-}
-
-uint64_t workspace_words(uint64_t nbuckets, uint64_t tiles) {
-    return nbuckets * (kHistWords + kStateWords + 2 * tiles);
 }
 
 bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geometry* g) {
@@ -362,6 +942,12 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     g->tiles = (uint32_t)((bucket_elems + kTile - 1) / kTile);
     g->k_full = mccl_hip_topk_k(bucket_elems, ratio);
     g->k_last = mccl_hip_topk_k(n_total - (nb - 1) * bucket_elems, ratio);
+    g->etiles = (uint32_t)((bucket_elems + kETile - 1) / kETile);
+    g->bwords = g->etiles * (kETile / 32);
+    // candidate capacity: 4 k + 4096 + n/256 entries per bucket, never more than the bucket
+    uint64_t cap = 4 * (uint64_t)g->k_full + 4096 + bucket_elems / 256;
+    if (cap > bucket_elems + kNSub) cap = bucket_elems + kNSub;
+    g->lsub = (uint32_t)((cap + kNSub - 1) / kNSub);
     return true;
 }
 
@@ -383,10 +969,11 @@ uint64_t mccl_hip_topk_max_compressed_size(uint64_t nbytes, double ratio) {
     return 4u + (uint64_t)k * 8u;
 }
 
-uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems) {
+uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, double ratio) {
     Geometry g;
-    if (!make_geometry(n_total, bucket_elems, 0.5, &g)) return 0;
-    return workspace_words(g.nbuckets, g.tiles) * 4 + 256;
+    if (!(ratio > 0.0 && ratio <= 1.0)) return 0;
+    if (!make_geometry(n_total, bucket_elems, ratio, &g)) return 0;
+    return workspace_words(g) * 4 + 256;
 }
 
 int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
@@ -400,34 +987,60 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     if ((wire_stride & 3) || ((uintptr_t)wire & 3)) return MCCL_HIP_ERR_ARG;
     const uint32_t kmax = g.k_full > g.k_last ? g.k_full : g.k_last;
     if (wire_stride < 4 + 8 * (uint64_t)kmax) return MCCL_HIP_ERR_CAPACITY;
-    if (workspace_bytes < workspace_words(g.nbuckets, g.tiles) * 4) return MCCL_HIP_ERR_WORKSPACE;
-    if ((uintptr_t)workspace & 3) return MCCL_HIP_ERR_ARG;
+    if (workspace_bytes < workspace_words(g) * 4 + 16) return MCCL_HIP_ERR_WORKSPACE;
     int rc = mccl_hip_init();
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    Workspace w = carve(workspace, g);
-
-    const uint64_t zero_words = (uint64_t)g.nbuckets * (kHistWords + kStateWords);
-    k_zero_words<<<clamp_u32((zero_words + kBlock - 1) / kBlock, 1, 1024), kBlock, 0, st>>>(w.hist, zero_words);
+    // the carved arrays are 16-byte aligned inside the caller's buffer
+    void* aligned = (void*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
+    Workspace w = carve(aligned, g);
+    const int path = tuning().topk_path;  // 0 auto, 1 exact path only, 2 fast path at any size
+    const bool fits = (uint64_t)g.etiles <= (uint64_t)kMarkTiles * kNSub;  // mark keeps a sub-list's bitmap in LDS
+    const bool fast = fits && (path == 2 || (path == 0 && g.bucket_elems >= kFastMinBucket));
 
     const uint64_t cap = (uint64_t)device_info().num_cus * (uint64_t)tuning().fold_blocks_per_cu;
     const uint64_t nvec = g.bucket_elems / 4;
-    uint64_t bx = (cap + g.nbuckets - 1) / g.nbuckets;
-    const uint64_t need_a = (nvec + kBlock * 2 - 1) / (kBlock * 2);
-    const uint32_t bx_a = clamp_u32(bx < need_a ? bx : need_a, 1, 65535);
+    const uint64_t bx = (cap + g.nbuckets - 1) / g.nbuckets;
     const uint64_t need_r = (nvec + kBlock * 4 - 1) / (kBlock * 4);
     const uint32_t bx_r = clamp_u32(bx < need_r ? bx : need_r, 1, 65535);
-
-    k_topk_pass_a<<<dim3(bx_a, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
-    k_topk_pick<kBins0><<<g.nbuckets, kBlock, 0, st>>>(g, w, 0);
-    k_topk_refine<<<dim3(bx_r, g.nbuckets), kBlock, 0, st>>>(residual, g, w, 1);
-    k_topk_pick<kBinsR><<<g.nbuckets, kBlock, 0, st>>>(g, w, 1);
-    k_topk_refine<<<dim3(bx_r, g.nbuckets), kBlock, 0, st>>>(residual, g, w, 2);
-    k_topk_pick<kBinsR><<<g.nbuckets, kBlock, 0, st>>>(g, w, 2);
-    k_topk_count<<<dim3(g.tiles, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
-    k_topk_scan<<<g.nbuckets, kBlock, 0, st>>>(g, w);
-    k_topk_emit<<<dim3(g.tiles, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
+    const uint32_t bx_t = clamp_u32(bx < g.tiles ? bx : g.tiles, 1, 65535);
+    if (fast) {
+        k_topk_sample<<<g.nbuckets, kSelThreads, 0, st>>>(grad, residual, g, w);
+        const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
+        k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
+        k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
+        k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
+        k_topk_mark<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
+        k_topk_emit_fast<<<dim3(g.etiles, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
+    } else {
+        const uint64_t zw = zeroed_words(g);
+        k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);
+        const uint64_t need_a = (nvec + kBlock * 2 - 1) / (kBlock * 2);
+        const uint32_t bx_a = clamp_u32(bx < need_a ? bx : need_a, 1, 65535);
+        k_topk_pass_a<<<dim3(bx_a, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
+        k_topk_refine<<<dim3(bx_r, g.nbuckets), kBlock, 0, st>>>(residual, g, w, 1, 0);
+        k_topk_refine<<<dim3(bx_r, g.nbuckets), kBlock, 0, st>>>(residual, g, w, 2, 0);
+        k_topk_count<<<dim3(bx_t, g.nbuckets), kBlock, 0, st>>>(residual, g, w, 0);
+        k_topk_emit<<<dim3(bx_t, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride, 0);
+    }
     return launch_status();
+}
+
+int mccl_hip_topk_path_report(const void* workspace, uint64_t n_total, uint64_t bucket_elems, double ratio,
+                              uint32_t* host_single_pass_buckets, uint32_t* host_buckets, void* stream) {
+    if (!workspace || !host_single_pass_buckets || !host_buckets) return MCCL_HIP_ERR_ARG;
+    Geometry g;
+    if (!(ratio > 0.0 && ratio <= 1.0) || !make_geometry(n_total, bucket_elems, ratio, &g)) return MCCL_HIP_ERR_ARG;
+    void* aligned = (void*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
+    Workspace w = carve(aligned, g);
+    std::vector<uint32_t> st((size_t)g.nbuckets * kStateWords);
+    MCCLHIP_TRY(hipMemcpyAsync(st.data(), w.state, st.size() * 4, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    MCCLHIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    uint32_t ok = 0;
+    for (uint32_t b = 0; b < g.nbuckets; b++) ok += st[(size_t)b * kStateWords + S_OK] ? 1u : 0u;
+    *host_single_pass_buckets = ok;
+    *host_buckets = g.nbuckets;
+    return MCCL_HIP_OK;
 }
 
 }  // extern "C"

@@ -99,8 +99,8 @@ def topk_wire_stride(bucket_elems: int, ratio: float) -> int:
     return topk_max_compressed_size(bucket_elems * 4, ratio)
 
 
-def topk_workspace(n_total: int, bucket_elems: int, device) -> torch.Tensor:
-    nbytes = int(_lib.load().mccl_hip_topk_workspace_bytes(n_total, bucket_elems))
+def topk_workspace(n_total: int, bucket_elems: int, ratio: float, device) -> torch.Tensor:
+    nbytes = int(_lib.load().mccl_hip_topk_workspace_bytes(n_total, bucket_elems, ratio))
     if nbytes == 0:
         raise _lib.MCCLHipError(-6, "topk_workspace_bytes")
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -120,12 +120,21 @@ def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
     if wire is None:
         wire = torch.empty(nb * stride, dtype=torch.uint8, device=grad.device)
     if workspace is None:
-        workspace = topk_workspace(max(n, 1), be, grad.device)
+        workspace = topk_workspace(max(n, 1), be, ratio, grad.device)
     rc = _lib.load().mccl_hip_topk_compress(grad.data_ptr(), residual.data_ptr(), n, be, ratio,
                                            wire.data_ptr(), stride, workspace.data_ptr(),
                                            workspace.numel(), _stream())
     _lib.check(rc, "topk_compress")
     return wire, stride
+
+
+def topk_path_report(workspace: torch.Tensor, n_total: int, bucket_elems: int, ratio: float):
+    """(buckets finished by the single-pass path, buckets) of the last compress call."""
+    ok, nb = C.c_uint32(0), C.c_uint32(0)
+    rc = _lib.load().mccl_hip_topk_path_report(workspace.data_ptr(), n_total, bucket_elems, ratio,
+                                               C.byref(ok), C.byref(nb), _stream())
+    _lib.check(rc, "topk_path_report")
+    return int(ok.value), int(nb.value)
 
 
 def topk_decompress(wire: torch.Tensor, wire_bytes: int, count: int,

@@ -41,7 +41,7 @@ def test_host_only_entry_points_agree_with_the_reference_formulas():
     assert lib.mccl_hip_topk_k(10, 0.01) == 1
     assert lib.mccl_hip_topk_max_compressed_size(6_553_600 * 4, 0.01) == 4 + 8 * 65_537
     assert lib.mccl_hip_strerror(-5) == b"TopK decompress: index out of bounds"
-    assert lib.mccl_hip_topk_workspace_bytes(96_510_024, 6_553_600) > 0
+    assert lib.mccl_hip_topk_workspace_bytes(96_510_024, 6_553_600, 0.01) > 0
     assert lib.mccl_hip_set_tuning(b"fold_blocks_per_cu", 4) == 0
     assert lib.mccl_hip_get_tuning(b"fold_blocks_per_cu") == 4
     assert lib.mccl_hip_set_tuning(b"fold_blocks_per_cu", 8) == 0

@@ -32,20 +32,28 @@ def oracle_buckets(g, r, ratio, be):
     return wires, res
 
 
+PATHS = {"exact": 1, "single-pass": 2}  # both must give the oracle's bytes on every input
+
+
 def check_compress(ops, g, r, ratio, be=None, pad=0):
     n = g.size
     be = be or n
     want_wires, want_res = oracle_buckets(g, r, ratio, be)
-    dg = to_dev(g, F32, pad); dr = to_dev(r, F32, pad)
-    wire, stride = ops.topk_compress(dg, dr, ratio, bucket_elems=be)
-    torch.cuda.synchronize()
-    got_res = to_np(dr, F32)
-    assert np.array_equal(bits(got_res), bits(want_res))
-    assert np.array_equal(to_np(dg, F32), g)  # gradient untouched
-    w = wire.cpu().numpy()
-    for b, ww in enumerate(want_wires):
-        got = w[b * stride: b * stride + ww.size]
-        assert got.tobytes() == ww.tobytes(), f"bucket {b}"
+    try:
+        for name, path in PATHS.items():
+            ops.set_tuning("topk_path", path)
+            dg = to_dev(g, F32, pad); dr = to_dev(r, F32, pad)
+            wire, stride = ops.topk_compress(dg, dr, ratio, bucket_elems=be)
+            torch.cuda.synchronize()
+            got_res = to_np(dr, F32)
+            assert np.array_equal(bits(got_res), bits(want_res)), name
+            assert np.array_equal(to_np(dg, F32), g), name  # gradient untouched
+            w = wire.cpu().numpy()
+            for b, ww in enumerate(want_wires):
+                got = w[b * stride: b * stride + ww.size]
+                assert got.tobytes() == ww.tobytes(), f"{name}: bucket {b}"
+    finally:
+        ops.set_tuning("topk_path", 0)
     return wire, stride, want_wires
 
 
@@ -80,6 +88,28 @@ def test_compress_degenerate_inputs(ops):
     check_compress(ops, np.tile(big, 1000), np.zeros(7000, np.float32), 0.3)
 
 
+def test_single_pass_path_on_clustered_and_tied_inputs(ops):
+    """Inputs that stress the candidate machinery: all large values in one corner
+    (sub-list overflow -> per-bucket fallback), a threshold shared by thousands of
+    equal keys (tie-break by index), and a bucket whose sample misleads."""
+    rng = np.random.default_rng(77)
+    n = 600_000
+    g = student_t(rng, n, ties=0.0) * np.float32(1e-3)
+    g[:20_000] = student_t(rng, 20_000, ties=0.0) * np.float32(10.0)     # clustered picks
+    check_compress(ops, g, np.zeros(n, np.float32), 0.01)
+    g = student_t(rng, n, ties=0.0)
+    thr = np.sort(np.abs(g))[-6000]
+    tie_pos = rng.choice(n, 5000, replace=False)
+    g[tie_pos] = thr * np.where(rng.random(5000) < 0.5, -1, 1).astype(np.float32)   # 5000 keys == T
+    check_compress(ops, g, np.zeros(n, np.float32), 0.01)
+    g = np.zeros(n, np.float32)
+    g[::512 * 4] = 1.0                      # the sample sees only these
+    g[1::7] = 2.0
+    check_compress(ops, g, np.zeros(n, np.float32), 0.01)
+    check_compress(ops, student_t(rng, n), (rng.standard_normal(n) * 1e-4).astype(np.float32), 0.001)
+    check_compress(ops, student_t(rng, n), np.zeros(n, np.float32), 0.3, be=300_000)
+
+
 def test_compress_many_buckets_short_last(ops):
     rng = np.random.default_rng(8)
     n, be = 1_000_003, 131_072
@@ -95,13 +125,15 @@ def test_config4_full_bucket_and_error_feedback_over_steps(ops):
     rng = np.random.default_rng(2024)
     res_o = np.zeros(n, np.float32)
     dres = to_dev(res_o, F32)
-    ws = ops.topk_workspace(n, n, DEV)
-    for step in range(2):
+    ws = ops.topk_workspace(n, n, 0.01, DEV)
+    for step in range(3):
         g = student_t(rng, n, ties=0.01)
         w, rc = oracle.topk_compress(g, res_o, 0.01)
         wire, stride = ops.topk_compress(to_dev(g, F32), dres, 0.01, workspace=ws)
         assert wire.cpu().numpy()[:rc].tobytes() == w.tobytes(), step
         assert np.array_equal(bits(to_np(dres, F32)), bits(res_o)), step
+        # this is the workload the single-pass path is built for: it must have taken it
+        assert ops.topk_path_report(ws, n, n, 0.01) == (1, 1), step
     assert oracle.parse_wire(w)[0] == 65_536
 
 
