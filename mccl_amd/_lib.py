@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmccl_hip.so")
+# MCCL_HIP_LIBRARY selects another build of the same ABI (kernel tuning experiments)
+LIB_PATH = os.environ.get("MCCL_HIP_LIBRARY") or os.path.join(_HERE, "libmccl_hip.so")
 
 # (restype, argtypes) for every symbol include/mccl_hip.h declares
 _vp, _u64, _u32, _i32, _f32, _f64 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int, C.c_float, C.c_double

@@ -26,10 +26,11 @@
 //              to the exact fallback), finishes the radix select on the second
 //              list: exact threshold key T, how many keys equal to T are taken
 //              and - when not all of them are - the largest index still taken
-//   mark       sets one bit per pick in a bitmap of the bucket
-//   ecount     picks per 8192-element emission tile (popcount)
-//   emit       ordered compaction of the bitmap: index order comes for free;
-//              values are gathered from the residual, which is zeroed there
+//   mark       one block per candidate sub-list (= a fixed set of 8192-element
+//              tiles): pick bitmaps of its tiles in LDS, each pick's rank inside
+//              its tile by popcount prefix, picks written per tile in index
+//              order to a staging list, residual zeroed at the picks
+//   emit       concatenates the tiles' runs in tile order into the payload
 // EXACT PATH (any input; also the per-bucket fallback of the fast path):
 //   [pass A]   residual <- grad + residual, histogram of key[30:20]
 //   refine x2  histograms of key[19:10], key[9:0] among prefix matches
@@ -53,13 +54,20 @@ constexpr int kBins0 = 2048;   // key[30:20]
 constexpr int kBinsR = 1024;   // key[19:10], key[9:0]
 constexpr int kHistWords = kBins0 + 2 * kBinsR;
 constexpr int kStateWords = 32;
-constexpr int kATile = 8192;   // fast path: elements per pass-A block
+#ifndef MCCLHIP_ATILE
+#define MCCLHIP_ATILE 8192
+#endif
+#ifndef MCCLHIP_AUNROLL
+#define MCCLHIP_AUNROLL 2
+#endif
+constexpr int kATile = MCCLHIP_ATILE;   // fast path: elements per pass-A block
 constexpr int kETile = 8192;   // fast path: elements per emission block (256 bitmap words, one per thread)
+static_assert(kATile == kETile, "a candidate sub-list must hold whole emission tiles");
 constexpr int kNSub = 64;      // fast path: candidate sub-lists per bucket
-constexpr int kStage = 512;    // fast path: staged candidates per wavefront
+constexpr int kStage = 384;    // fast path: staged candidates per wavefront (>= 256: one vector's worth)
 constexpr int kSelThreads = 1024;
 constexpr uint64_t kFastMinBucket = 1u << 18;
-constexpr int kMarkTiles = 48;  // fast path: emission tiles one mark block can hold in LDS
+constexpr int kMarkTiles = 24;  // fast path: emission tiles one mark block can hold in LDS
 constexpr int kSample = 12288;  // fast path: sampled elements per bucket (12 per select thread)
 
 // per-bucket state words
@@ -84,7 +92,6 @@ struct Geometry {
     uint32_t k_full;   // k of a bucket with bucket_elems elements
     uint32_t k_last;   // k of the last bucket
     uint32_t etiles;   // emission tiles per bucket
-    uint32_t bwords;   // bitmap words per bucket (etiles * 256)
     uint32_t lsub;     // capacity of one candidate sub-list (entries)
 };
 
@@ -95,12 +102,12 @@ struct Workspace {
     uint32_t* state;        // [nbuckets][kStateWords]
     uint32_t* sub_count;    // [nbuckets][kNSub]
     uint32_t* etile_count;  // [nbuckets][etiles]
-    uint32_t* bitmap;       // [nbuckets][bwords]
+    uint32_t* etile_off;    // [nbuckets][etiles]  start of the tile's run inside its sub-list's staging
     // scratch, written before read
     uint32_t* tile_gt;      // [nbuckets][tiles]
     uint32_t* tile_eq;      // [nbuckets][tiles]
     uint32_t* list;         // [nbuckets][kNSub][lsub][2]  (index, bits)
-    uint32_t* list2;        // [nbuckets][kNSub * lsub][2] candidates of the threshold bin
+    uint32_t* list2;        // [nbuckets][kNSub * lsub][2] candidates of the threshold bin, later the staged picks
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -448,13 +455,15 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     const float* rp = residual + (uint64_t)b * g.bucket_elems;
     const uint64_t nvec = bn / 4;
     constexpr int SV = kSample / 4;  // sampled vectors
-    const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)nvec : (uint32_t)SV;
-    const uint64_t stride = nsv ? nvec / nsv : 1;
+    // sampled in runs of 8 vectors (one 128-byte line per array), runs evenly spread
+    const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)(nvec & ~7ull) : (uint32_t)SV;
+    const uint64_t stride = nsv ? (nvec / (nsv / 8)) : 8;  // vectors between run starts (>= 8)
     u4a gv[SV / kSelThreads], rv[SV / kSelThreads];
 #pragma unroll
     for (int j = 0; j < SV / kSelThreads; j++) {
         const uint32_t i = (uint32_t)j * kSelThreads + threadIdx.x;
-        const uint64_t v = (uint64_t)(i < nsv ? i : 0) * stride;
+        const uint32_t ii = i < nsv ? i : 0;
+        const uint64_t v = (uint64_t)(ii >> 3) * stride + (ii & 7);
         gv[j] = nsv ? *(const u4u4*)(gp + v * 4) : u4a{0u, 0u, 0u, 0u};
         rv[j] = nsv ? *(const u4u4*)(rp + v * 4) : u4a{0u, 0u, 0u, 0u};
     }
@@ -526,13 +535,32 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
     const uint64_t bn = bucket_count(g, b);
     const uint64_t e0 = (uint64_t)t * kATile;
     if (e0 >= bn) return;
-    for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
-    __syncthreads();
     const float* gp = grad + (uint64_t)b * g.bucket_elems;
     float* rp = residual + (uint64_t)b * g.bucket_elems;
+    constexpr int U = MCCLHIP_AUNROLL;
+    constexpr int ROUNDS = kATile / (kBlock * 4 * U);
+    const uint64_t tile_end = (e0 + kATile) < bn ? (e0 + kATile) : bn;
+    const uint64_t nfull = (tile_end - e0) / 4;  // full vectors in this tile
+    // The streaming loads of a round are issued one round ahead: round 0's before
+    // the block's set-up (LDS clear, bucket parameters), round r+1's before round r
+    // is processed, so the set-up latencies hide behind the HBM latency.
+    u4a gv[ROUNDS][U], rv[ROUNDS][U];
+    auto issue = [&](int round) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint64_t vi = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
+            if (vi < nfull) {
+                gv[round][u] = __builtin_nontemporal_load((const u4u4*)(gp + e0 + vi * 4));
+                rv[round][u] = __builtin_nontemporal_load((const u4u4*)(rp + e0 + vi * 4));
+            }
+        }
+    };
+    issue(0);
+    for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
     const uint32_t lo_key = w.state[(uint64_t)b * kStateWords + S_LO_KEY];
     const uint32_t hi_key = w.state[(uint64_t)b * kStateWords + S_HI_KEY];
     const uint32_t wshift = w.state[(uint64_t)b * kStateWords + S_SHIFT];
+    __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const uint32_t sub = t % kNSub;
@@ -554,34 +582,23 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         staged = 0;
     };
 
-    constexpr int U = 4;
-    const uint64_t tile_end = (e0 + kATile) < bn ? (e0 + kATile) : bn;
-    const uint64_t nfull = (tile_end - e0) / 4;  // full vectors in this tile
-#pragma unroll 1
-    for (int round = 0; round < kATile / (kBlock * 4 * U); round++) {
-        u4a gv[U], rv[U];
-        uint64_t vi[U];
+#pragma unroll
+    for (int round = 0; round < ROUNDS; round++) {
+        if (round + 1 < ROUNDS) issue(round + 1);
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            vi[u] = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
-            if (vi[u] < nfull) {
-                gv[u] = __builtin_nontemporal_load((const u4u4*)(gp + e0 + vi[u] * 4));
-                rv[u] = __builtin_nontemporal_load((const u4u4*)(rp + e0 + vi[u] * 4));
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
+            const uint64_t vi = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
             u4a a = {0u, 0u, 0u, 0u};
             bool cand[4] = {false, false, false, false};
-            const bool live = vi[u] < nfull;
+            const bool live = vi < nfull;
             if (live) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const float adj = u2f(gv[u][q]) + u2f(rv[u][q]);
+                    const float adj = u2f(gv[round][u][q]) + u2f(rv[round][u][q]);
                     a[q] = f2u(adj);
                     cand[q] = key_of(adj) >= lo_key;
                 }
-                __builtin_nontemporal_store(a, (u4u4*)(rp + e0 + vi[u] * 4));
+                __builtin_nontemporal_store(a, (u4u4*)(rp + e0 + vi * 4));
             }
             const bool any = cand[0] | cand[1] | cand[2] | cand[3];
             if (__ballot(any)) {  // wave-uniform
@@ -591,7 +608,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
                     const uint64_t m = __ballot(cand[q]);
                     if (cand[q]) {
                         const uint32_t pos = staged + __popcll(m & ((1ull << lane) - 1ull));
-                        stage[wave][pos][0] = (uint32_t)(e0 + vi[u] * 4 + q);
+                        stage[wave][pos][0] = (uint32_t)(e0 + vi * 4 + q);
                         stage[wave][pos][1] = a[q];
                         atomicAdd(&lh[window_bin(a[q] & 0x7FFFFFFFu, lo_key, hi_key, wshift)], 1u);
                     }
@@ -828,11 +845,16 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
 }
 
 // One block per candidate sub-list.  A sub-list holds the candidates of the
-// pass-A tiles t = s, s + kNSub, ...; an emission tile is the same 8192 elements,
-// so this block owns those tiles' bitmap words outright: it builds them in LDS,
-// stores them whole (no atomics, no pre-zeroed bitmap) and counts their picks.
-__global__ __launch_bounds__(kBlock) void k_topk_mark(Geometry g, Workspace w) {
+// pass-A tiles t = s, s + kNSub, ..., so this block sees every pick of those
+// 8192-element tiles.  It builds the tiles' pick bitmaps in LDS, derives every
+// pick's rank inside its tile from them (popcount prefix), writes the picks of
+// each tile, in index order, as one contiguous run of the bucket's staging
+// list, zeroes the residual at the picks, and records (offset, count) per tile.
+// The emit kernel then only concatenates the runs.
+__global__ __launch_bounds__(kBlock) void k_topk_mark(float* residual, Geometry g, Workspace w) {
     __shared__ uint32_t bm[kMarkTiles * (kETile / 32)];
+    __shared__ uint32_t pre[kMarkTiles * (kETile / 32)];  // picks of the tile before this word
+    __shared__ uint32_t tcount[kMarkTiles], toff[kMarkTiles];
     const uint32_t b = blockIdx.y, s = blockIdx.x;
     const uint32_t* st = w.state + (uint64_t)b * kStateWords;
     if (!st[S_OK]) return;
@@ -849,8 +871,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_mark(Geometry g, Workspace w) {
         for (int j = 0; j < 8; j++) {
             const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
             if (c.valid[j] && (key > T || (key == T && c.idx[j] <= istar))) {
-                const uint32_t tile = c.idx[j] / kETile;            // == s (mod kNSub)
-                const uint32_t word = (tile / kNSub) * (kETile / 32) + ((c.idx[j] % kETile) >> 5);
+                const uint32_t word = (c.idx[j] / kETile / kNSub) * (kETile / 32) + ((c.idx[j] % kETile) >> 5);
                 atomicOr(&bm[word], 1u << (c.idx[j] & 31));
             }
         }
@@ -858,44 +879,66 @@ __global__ __launch_bounds__(kBlock) void k_topk_mark(Geometry g, Workspace w) {
     __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
     for (uint32_t j = threadIdx.x / kWave; j < ntiles; j += kBlock / kWave) {  // one wavefront per tile
-        const uint32_t tile = s + j * kNSub;
         const u4a v = ((const u4a*)(bm + j * (kETile / 32)))[lane];
-        ((u4a*)(w.bitmap + (uint64_t)b * g.bwords + (uint64_t)tile * (kETile / 32)))[lane] = v;
-        uint32_t c = __popc(v[0]) + __popc(v[1]) + __popc(v[2]) + __popc(v[3]);
+        const uint32_t c0 = __popc(v[0]), c1 = __popc(v[1]), c2 = __popc(v[2]), c3 = __popc(v[3]);
+        const uint32_t inc = wave_inclusive_scan(c0 + c1 + c2 + c3);
+        const uint32_t ex = inc - (c0 + c1 + c2 + c3);
+        u4a p = {ex, ex + c0, ex + c0 + c1, ex + c0 + c1 + c2};
+        ((u4a*)(pre + j * (kETile / 32)))[lane] = p;
+        if (lane == kWave - 1) tcount[j] = inc;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t run = 0;
+        for (uint32_t j = 0; j < ntiles; j++) { toff[j] = run; run += tcount[j]; }
+    }
+    __syncthreads();
+    if (threadIdx.x < ntiles) {
+        const uint32_t tile = s + threadIdx.x * kNSub;
+        w.etile_count[(uint64_t)b * g.etiles + tile] = tcount[threadIdx.x];
+        w.etile_off[(uint64_t)b * g.etiles + tile] = toff[threadIdx.x];
+    }
+    uint32_t* stg = w.list2 + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
+        const EntryChunk c = load_entries(l, base, cnt);
 #pragma unroll
-        for (int d = kWave / 2; d > 0; d >>= 1) c += __shfl_xor(c, d, kWave);
-        if (lane == 0) w.etile_count[(uint64_t)b * g.etiles + tile] = c;
+        for (int j = 0; j < 8; j++) {
+            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
+            if (c.valid[j] && (key > T || (key == T && c.idx[j] <= istar))) {
+                const uint32_t tj = c.idx[j] / kETile / kNSub;
+                const uint32_t word = tj * (kETile / 32) + ((c.idx[j] % kETile) >> 5);
+                const uint32_t rank = pre[word] + __popc(bm[word] & ((1u << (c.idx[j] & 31)) - 1u));
+                const uint32_t pos = toff[tj] + rank;
+                stg[2 * (uint64_t)pos] = c.idx[j];
+                stg[2 * (uint64_t)pos + 1] = c.bits[j];
+                rp[c.idx[j]] = 0.0f;
+            }
+        }
     }
 }
 
-// Ordered compaction of the bitmap: 256 words per block, one per thread.
-__global__ __launch_bounds__(kBlock) void k_topk_emit_fast(float* residual, Geometry g, Workspace w,
-                                                           uint8_t* wire, uint64_t wire_stride) {
-    __shared__ uint32_t smem[kBlock / kWave + 2];
-    const uint32_t b = blockIdx.y, t = blockIdx.x;
-    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    if (!st[S_OK]) return;
-    const uint64_t bn = bucket_count(g, b);
-    if ((uint64_t)t * kETile >= bn) return;
+// Concatenates the tiles' runs in tile order: one wavefront per tile.
+__global__ __launch_bounds__(kBlock) void k_topk_emit_fast(Geometry g, Workspace w, uint8_t* wire,
+                                                           uint64_t wire_stride) {
+    const uint32_t b = blockIdx.y;
+    if (!w.state[(uint64_t)b * kStateWords + S_OK]) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t t = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
     uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
-    if (t == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    if (t == 0 && lane == 0) out[0] = bucket_k(g, b);
+    if (t >= g.etiles) return;
     const uint32_t* ec = w.etile_count + (uint64_t)b * g.etiles;
-    uint32_t before = 0;
-    for (uint32_t i = threadIdx.x; i < t; i += kBlock) before += ec[i];
-    uint32_t base;
-    block_exclusive_scan(before, smem, &base);
-    uint32_t m = w.bitmap[(uint64_t)b * g.bwords + (uint64_t)t * (kETile / 32) + threadIdx.x];
-    uint32_t total;
-    uint32_t pos = base + block_exclusive_scan((uint32_t)__popc(m), smem, &total);
-    while (m) {
-        const int bit = __ffs(m) - 1;
-        m &= m - 1;
-        const uint32_t idx = t * (uint32_t)kETile + threadIdx.x * 32u + (uint32_t)bit;
-        out[1 + 2 * (uint64_t)pos] = idx;
-        out[2 + 2 * (uint64_t)pos] = f2u(rp[idx]);
-        rp[idx] = 0.0f;
-        pos++;
+    const uint32_t cnt = ec[t];
+    const uint32_t off = w.etile_off[(uint64_t)b * g.etiles + t];
+    uint32_t base = 0;
+    for (uint32_t i = lane; i < t; i += kWave) base += ec[i];
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) base += __shfl_xor(base, d, kWave);
+    const uint32_t* src = w.list2 + ((((uint64_t)b * kNSub + (t % kNSub)) * g.lsub) + off) * 2;
+    for (uint32_t i = lane; i < cnt; i += kWave) {
+        out[1 + 2 * (uint64_t)(base + i)] = src[2 * (uint64_t)i];
+        out[2 + 2 * (uint64_t)(base + i)] = src[2 * (uint64_t)i + 1];
     }
 }
 
@@ -909,7 +952,7 @@ uint64_t zeroed_words(const Geometry& g) {
 }
 
 uint64_t workspace_words(const Geometry& g) {
-    return zeroed_words(g) + align4((uint64_t)g.nbuckets * g.etiles) + align4((uint64_t)g.nbuckets * g.bwords) +
+    return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.etiles) +
            2 * align4((uint64_t)g.nbuckets * g.tiles) +
            2 * align4((uint64_t)g.nbuckets * kNSub * g.lsub * 2);
 }
@@ -922,7 +965,7 @@ Workspace carve(void* base, const Geometry& g) {
     w.state = p;       p += align4((uint64_t)g.nbuckets * kStateWords);
     w.sub_count = p;   p += align4((uint64_t)g.nbuckets * kNSub);
     w.etile_count = p; p += align4((uint64_t)g.nbuckets * g.etiles);
-    w.bitmap = p;      p += align4((uint64_t)g.nbuckets * g.bwords);
+    w.etile_off = p;   p += align4((uint64_t)g.nbuckets * g.etiles);
     w.tile_gt = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
     w.tile_eq = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
     w.list = p;        p += align4((uint64_t)g.nbuckets * kNSub * g.lsub * 2);
@@ -943,7 +986,6 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     g->k_full = mccl_hip_topk_k(bucket_elems, ratio);
     g->k_last = mccl_hip_topk_k(n_total - (nb - 1) * bucket_elems, ratio);
     g->etiles = (uint32_t)((bucket_elems + kETile - 1) / kETile);
-    g->bwords = g->etiles * (kETile / 32);
     // candidate capacity: 4 k + 4096 + n/256 entries per bucket, never more than the bucket
     uint64_t cap = 4 * (uint64_t)g->k_full + 4096 + bucket_elems / 256;
     if (cap > bucket_elems + kNSub) cap = bucket_elems + kNSub;
@@ -1010,8 +1052,8 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
         k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
         k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
-        k_topk_mark<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
-        k_topk_emit_fast<<<dim3(g.etiles, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
+        k_topk_mark<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
+        k_topk_emit_fast<<<dim3((g.etiles + 3) / 4, g.nbuckets), kBlock, 0, st>>>(g, w, (uint8_t*)wire, wire_stride);
     } else {
         const uint64_t zw = zeroed_words(g);
         k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);
