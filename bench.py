@@ -217,8 +217,9 @@ def main() -> int:
         status = torch.zeros(1, dtype=torch.int32, device=dev)
         acc = torch.empty(N, device=dev)
         acc_bytes = 4 * N + 8 * sum(ks) * W
+        sws = ops.sparse_workspace(N, BUCKET, W, dev)
         sa = stats(gpu_time(lambda: ops.sparse_accumulate(acc, wires, stride, bucket_elems=BUCKET,
-                                                          scale_by=0.125, status=status))[1])
+                                                          scale_by=0.125, status=status, workspace=sws))[1])
         extra["config5_sparse_accumulate"] = {"ms": sa["avg_ms"], "GBps": rate(acc_bytes, sa["avg_ms"]),
                                               "frac": rate(acc_bytes, sa["avg_ms"]) / HBM_PEAK_GBPS,
                                               "bytes": acc_bytes, "status": int(status)}

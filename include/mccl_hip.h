@@ -182,7 +182,13 @@ int mccl_hip_topk_decompress(const void* wire, uint64_t wire_bytes, float* dense
  * one payload must have ascending indices (what compress emits). */
 int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems,
                                const void* const* host_wires, int ws, uint64_t wire_stride,
-                               int apply_scale, float scale, int* status, void* stream);
+                               int apply_scale, float scale, int* status, void* workspace,
+                               uint64_t workspace_bytes, void* stream);
+/* Scratch for mccl_hip_sparse_accumulate (per rank and bucket, the position in
+ * the payload at which every 4096-element output tile begins).  Passing
+ * workspace = NULL is allowed: the ranges are then found by binary search in
+ * every block, which costs about 3x the time on MI355X. */
+uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, int ws);
 
 /* ---- ordering ----------------------------------------------------------- */
 

@@ -132,6 +132,143 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate(float* acc, uint64
     }
 }
 
+// ---- tile bounds pre-pass ------------------------------------------------------
+// start[(b * ws + r) * (tiles + 1) + t] = first pair of rank r's bucket-b payload
+// whose index lies in tile t or later; start[..][tiles] = k.  One thread per pair:
+// pair p writes the entry of every tile that begins between pair p-1 and pair p
+// (usually none), so each entry is written exactly once for a sorted payload.
+__global__ __launch_bounds__(kBlock) void k_sparse_bounds(WirePtrs wires, int ws, uint64_t wire_stride,
+                                                          uint64_t n_total, uint64_t bucket_elems, uint32_t tiles,
+                                                          uint32_t* start, int* status) {
+    const uint32_t b = blockIdx.y / (uint32_t)ws, r = blockIdx.y % (uint32_t)ws;
+    const uint64_t bstart = (uint64_t)b * bucket_elems;
+    const uint64_t bn = (n_total - bstart) < bucket_elems ? (n_total - bstart) : bucket_elems;
+    const uint32_t* wp = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride);
+    const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
+    uint32_t k = wp[0];
+    if (k > kmax) {
+        if (status) *status = MCCL_HIP_ERR_SIZE;
+        k = 0;
+    }
+    uint32_t* st = start + ((uint64_t)b * ws + r) * (tiles + 1);
+    constexpr int PP = 4;  // pairs per thread, all loads issued before the first use
+    const uint32_t p0 = blockIdx.x * (kBlock * PP) + threadIdx.x;
+    if (k == 0) {
+        for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t <= tiles; t += gridDim.x * kBlock) st[t] = 0;
+        return;
+    }
+    uint32_t idx[PP], prev[PP];
+#pragma unroll
+    for (int j = 0; j < PP; j++) {
+        const uint32_t p = p0 + (uint32_t)j * kBlock;
+        const uint32_t pc = p < k ? p : k - 1;
+        idx[j] = wp[1 + 2 * (uint64_t)pc];
+        prev[j] = wp[1 + 2 * (uint64_t)(pc > 0 ? pc - 1 : 0)];
+    }
+#pragma unroll
+    for (int j = 0; j < PP; j++) {
+        const uint32_t p = p0 + (uint32_t)j * kBlock;
+        if (p >= k) continue;
+        if (idx[j] >= bn && status) *status = MCCL_HIP_ERR_INDEX;
+        uint32_t t_hi = idx[j] / kAccTile;  // tiles (t_prev, t_hi] begin at pair p
+        if (t_hi > tiles) t_hi = tiles;
+        int64_t t_prev = -1;
+        if (p > 0) {
+            if (prev[j] >= idx[j] && status) *status = MCCL_HIP_ERR_INDEX;  // not ascending
+            t_prev = prev[j] / kAccTile;
+        }
+        for (int64_t t = t_prev + 1; t <= (int64_t)t_hi; t++) st[t] = p;
+        if (p == k - 1)
+            for (uint32_t t = t_hi + 1; t <= tiles; t++) st[t] = k;
+    }
+}
+
+// Accumulate with precomputed bounds: every block reads its 2 * ws bounds with one
+// load per lane, then issues the loads of all its pairs (every rank) before the
+// first LDS add; the adds run rank by rank.
+__global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint64_t n_total,
+                                                                uint64_t bucket_elems, WirePtrs wires, int ws,
+                                                                uint64_t wire_stride, uint32_t tiles,
+                                                                const uint32_t* start, int apply_scale,
+                                                                float scale, int* status) {
+    __shared__ float tile[kAccTile];
+    __shared__ uint32_t lo_s[MCCL_HIP_MAX_WORLD], hi_s[MCCL_HIP_MAX_WORLD];
+    const uint32_t b = blockIdx.y, t = blockIdx.x;
+    const uint64_t bstart = (uint64_t)b * bucket_elems;
+    const uint64_t bn = (n_total - bstart) < bucket_elems ? (n_total - bstart) : bucket_elems;
+    const uint64_t tstart = (uint64_t)t * kAccTile;
+    if (tstart >= bn) return;
+    const uint32_t tlen = (uint32_t)((bn - tstart) < kAccTile ? (bn - tstart) : kAccTile);
+    const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
+    if (threadIdx.x < 2 * ws) {
+        const int r = threadIdx.x < ws ? threadIdx.x : threadIdx.x - ws;
+        uint32_t v = start[((uint64_t)b * ws + r) * (tiles + 1) + t + (threadIdx.x < ws ? 0 : 1)];
+        if (v > kmax) v = kmax;  // stale bound of a malformed payload: stay inside the buffer
+        if (threadIdx.x < ws) lo_s[r] = v; else hi_s[r] = v;
+    }
+    for (int i = threadIdx.x; i < kAccTile; i += kBlock) tile[i] = 0.0f;
+    __syncthreads();
+    constexpr int RB = 8;  // ranks whose pairs are in flight together
+    for (int r0 = 0; r0 < ws; r0 += RB) {
+        uint32_t off[RB], val[RB];
+        bool have[RB], more = false;
+#pragma unroll
+        for (int j = 0; j < RB; j++) {
+            const int r = r0 + j;
+            have[j] = false;
+            if (r < ws) {
+                const uint32_t lo = lo_s[r], hi = hi_s[r];
+                const uint32_t p = lo + threadIdx.x;
+                if (hi > lo + kBlock) more = true;
+                if (p < hi) {
+                    const uint32_t* pairs = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride) + 1;
+                    off[j] = pairs[2 * (uint64_t)p] - (uint32_t)tstart;
+                    val[j] = pairs[2 * (uint64_t)p + 1];
+                    have[j] = true;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < RB; j++) {
+            const int r = r0 + j;
+            if (r < ws) {
+                if (have[j]) {
+                    if (off[j] < tlen) tile[off[j]] = tile[off[j]] + u2f(val[j]);
+                    else if (status) *status = MCCL_HIP_ERR_INDEX;
+                }
+                // dense tiles (more than kBlock pairs of one rank): the rest, still in rank order
+                if (__syncthreads_or(more ? 1 : 0)) {
+                    const uint32_t lo = lo_s[r], hi = hi_s[r];
+                    const uint32_t* pairs = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride) + 1;
+                    for (uint32_t p = lo + kBlock + threadIdx.x; p < hi; p += kBlock) {
+                        const uint32_t o = pairs[2 * (uint64_t)p] - (uint32_t)tstart;
+                        if (o < tlen) tile[o] = tile[o] + u2f(pairs[2 * (uint64_t)p + 1]);
+                        else if (status) *status = MCCL_HIP_ERR_INDEX;
+                    }
+                    __syncthreads();
+                }
+            }
+        }
+    }
+    float* out = acc + bstart + tstart;
+    if (tlen == kAccTile && (((uintptr_t)out & 15) == 0)) {
+        for (int i = threadIdx.x; i < kAccTile / 4; i += kBlock) {
+            u4a v;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float x = tile[4 * i + q];
+                v[q] = f2u(apply_scale ? x * scale : x);
+            }
+            __builtin_nontemporal_store(v, (u4a*)out + i);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < tlen; i += kBlock) {
+            const float x = tile[i];
+            out[i] = apply_scale ? x * scale : x;
+        }
+    }
+}
+
 }  // namespace
 }  // namespace mcclhip
 
@@ -158,27 +295,51 @@ int mccl_hip_topk_decompress(const void* wire, uint64_t wire_bytes, float* dense
     return launch_status();
 }
 
+uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, int ws) {
+    if (n_total == 0 || bucket_elems == 0 || ws < 1 || ws > MCCL_HIP_MAX_WORLD) return 0;
+    if (bucket_elems > n_total) bucket_elems = n_total;
+    const uint64_t nb = (n_total + bucket_elems - 1) / bucket_elems;
+    const uint64_t tiles = (bucket_elems + kAccTile - 1) / kAccTile;
+    return nb * (uint64_t)ws * (tiles + 1) * 4 + 64;
+}
+
 int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems,
                                const void* const* host_wires, int ws, uint64_t wire_stride,
-                               int apply_scale, float scale, int* status, void* stream) {
+                               int apply_scale, float scale, int* status, void* workspace,
+                               uint64_t workspace_bytes, void* stream) {
     if (!acc || !host_wires || ws < 1 || ws > MCCL_HIP_MAX_WORLD) return MCCL_HIP_ERR_ARG;
     if (n_total == 0 || n_total > MCCL_HIP_MAX_ELEMS || bucket_elems == 0) return MCCL_HIP_ERR_ARG;
     if (wire_stride < 4 || (wire_stride & 3)) return MCCL_HIP_ERR_ARG;
     if (bucket_elems > n_total) bucket_elems = n_total;
     if (bucket_elems > 0xFFFFFFFFull) return MCCL_HIP_ERR_ARG;
     const uint64_t nb = (n_total + bucket_elems - 1) / bucket_elems;
-    if (nb > 65535) return MCCL_HIP_ERR_ARG;
+    if (nb * (uint64_t)ws > 65535) return MCCL_HIP_ERR_ARG;
     WirePtrs wp;
     for (int r = 0; r < MCCL_HIP_MAX_WORLD; r++) wp.w[r] = nullptr;
     for (int r = 0; r < ws; r++) {
         if (!host_wires[r] || ((uintptr_t)host_wires[r] & 3)) return MCCL_HIP_ERR_ARG;
         wp.w[r] = (const uint8_t*)host_wires[r];
     }
+    if (workspace && workspace_bytes < mccl_hip_sparse_accumulate_workspace_bytes(n_total, bucket_elems, ws))
+        return MCCL_HIP_ERR_WORKSPACE;
     int rc = mccl_hip_init();
     if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
     const uint32_t tiles = (uint32_t)((bucket_elems + kAccTile - 1) / kAccTile);
-    k_sparse_accumulate<<<dim3(tiles, (uint32_t)nb), kBlock, 0, (hipStream_t)stream>>>(
-        acc, n_total, bucket_elems, wp, ws, wire_stride, apply_scale, scale, status);
+    if (!workspace) {
+        // no scratch: every block finds its ranges by binary search
+        k_sparse_accumulate<<<dim3(tiles, (uint32_t)nb), kBlock, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
+                                                                           wire_stride, apply_scale, scale, status);
+        return launch_status();
+    }
+    uint32_t* start = (uint32_t*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
+    const uint64_t kmax = (wire_stride - 4) / 8;
+    const uint32_t bx = clamp_u32((kmax + kBlock * 4 - 1) / (kBlock * 4), 1, 0x7FFFFFFF);
+    k_sparse_bounds<<<dim3(bx, (uint32_t)(nb * ws)), kBlock, 0, st>>>(wp, ws, wire_stride, n_total, bucket_elems,
+                                                                        tiles, start, status);
+    k_sparse_accumulate_b<<<dim3(tiles, (uint32_t)nb), kBlock, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
+                                                                         wire_stride, tiles, start, apply_scale,
+                                                                         scale, status);
     return launch_status();
 }
 

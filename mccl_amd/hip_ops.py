@@ -148,15 +148,28 @@ def topk_decompress(wire: torch.Tensor, wire_bytes: int, count: int,
     return dense
 
 
+def sparse_workspace(n_total: int, bucket_elems: int, ws: int, device) -> torch.Tensor:
+    nbytes = int(_lib.load().mccl_hip_sparse_accumulate_workspace_bytes(n_total, bucket_elems, ws))
+    if nbytes == 0:
+        raise _lib.MCCLHipError(-6, "sparse_accumulate_workspace_bytes")
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
 def sparse_accumulate(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_stride: int,
                       bucket_elems: Optional[int] = None, scale_by: Optional[float] = None,
-                      status: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      status: Optional[torch.Tensor] = None, workspace="auto") -> torch.Tensor:
+    """workspace: "auto" allocates the scratch, None selects the scratch-free kernel."""
     _dev(acc, "acc")
     n = acc.numel()
+    be = bucket_elems or max(n, 1)
+    if isinstance(workspace, str):
+        workspace = sparse_workspace(n, be, len(wires), acc.device)
     rc = _lib.load().mccl_hip_sparse_accumulate(
-        acc.data_ptr(), n, bucket_elems or max(n, 1), _ptrs(wires), len(wires), wire_stride,
+        acc.data_ptr(), n, be, _ptrs(wires), len(wires), wire_stride,
         0 if scale_by is None else 1, 0.0 if scale_by is None else scale_by,
-        None if status is None else status.data_ptr(), _stream())
+        None if status is None else status.data_ptr(),
+        None if workspace is None else workspace.data_ptr(), 0 if workspace is None else workspace.numel(),
+        _stream())
     _lib.check(rc, "sparse_accumulate")
     return acc
 

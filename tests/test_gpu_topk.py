@@ -176,10 +176,13 @@ def test_decompress_matches_oracle_and_reports_errors(ops):
         ops.topk_decompress(dw, rc - 3, n, dense=dense, status=status)
 
 
-@pytest.mark.parametrize("ws,n,be", [(8, 300_007, 65_536), (3, 4096, 4096), (2, 5, 5), (8, 1_000_000, 1_000_000)])
+@pytest.mark.parametrize("ws,n,be", [(8, 300_007, 65_536), (3, 4096, 4096), (2, 5, 5), (8, 1_000_000, 1_000_000),
+                                      (3, 20_000, 20_000), (12, 50_000, 16_384)])
 def test_sparse_accumulate_matches_dense_reference_form(ops, ws, n, be):
     rng = np.random.default_rng(ws + n)
     ratio = 0.01 if n > 1000 else 0.5
+    if n == 20_000:
+        ratio = 0.5  # more than 256 pairs of one rank per 4096-element tile
     nb = (n + be - 1) // be
     stride = ops.topk_wire_stride(be, ratio)
     # ~30 % of a rank's picks shared with other ranks: a common pool of large entries
@@ -202,10 +205,12 @@ def test_sparse_accumulate_matches_dense_reference_form(ops, ws, n, be):
         assert rc == oracle.OK
         want[s:e] = acc
     status = torch.zeros(1, dtype=torch.int32, device=DEV)
-    acc = torch.full((n,), 3.0, device=DEV)
-    ops.sparse_accumulate(acc, dev_wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status)
-    assert int(status) == 0
-    assert np.array_equal(bits(to_np(acc, F32)), bits(want))
+    for workspace in ("auto", None):   # with the tile-bounds scratch, and the scratch-free kernel
+        acc = torch.full((n,), 3.0, device=DEV)
+        ops.sparse_accumulate(acc, dev_wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status,
+                              workspace=workspace)
+        assert int(status) == 0
+        assert np.array_equal(bits(to_np(acc, F32)), bits(want)), workspace
 
 
 def test_sparse_accumulate_flags_bad_payloads(ops):
@@ -216,12 +221,19 @@ def test_sparse_accumulate_flags_bad_payloads(ops):
     good[4:20] = np.array([5, 0x3F800000, 9_999, 0x40000000], "<u4").view(np.uint8)
     status = torch.zeros(1, dtype=torch.int32, device=DEV)
     acc = torch.empty(n, device=DEV)
-    ops.sparse_accumulate(acc, [torch.from_numpy(good).to(DEV)], stride, status=status)
-    assert int(status) == 0 and float(acc[5]) == 1.0 and float(acc[9_999]) == 2.0 and float(acc.sum()) == 3.0
-    bad = good.copy(); bad[12:16] = np.array([10_000], "<u4").view(np.uint8)   # index == count
+    for workspace in ("auto", None):
+        status.zero_()
+        ops.sparse_accumulate(acc, [torch.from_numpy(good).to(DEV)], stride, status=status, workspace=workspace)
+        assert int(status) == 0 and float(acc[5]) == 1.0 and float(acc[9_999]) == 2.0 and float(acc.sum()) == 3.0
+        bad = good.copy(); bad[12:16] = np.array([10_000], "<u4").view(np.uint8)   # index == count
+        ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status, workspace=workspace)
+        assert int(status) == oracle.ERR_INDEX
+        status.zero_()
+        bad = good.copy(); bad[:4] = np.array([17], "<u4").view(np.uint8)           # k beyond the stride
+        ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status, workspace=workspace)
+        assert int(status) == oracle.ERR_SIZE
+    # descending indices: flagged, never out of bounds
+    status.zero_()
+    bad = good.copy(); bad[4:20] = np.array([9_999, 0x3F800000, 5, 0x40000000], "<u4").view(np.uint8)
     ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status)
     assert int(status) == oracle.ERR_INDEX
-    status.zero_()
-    bad = good.copy(); bad[:4] = np.array([17], "<u4").view(np.uint8)           # k beyond the stride
-    ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status)
-    assert int(status) == oracle.ERR_SIZE
