@@ -21,7 +21,7 @@ namespace mcclhip {
 
 namespace {
 
-constexpr int kAccTile = 4096;
+constexpr int kAccTile = 8192;  // output elements per block, accumulated in LDS (32 KiB)
 
 __global__ __launch_bounds__(kBlock) void k_fill_zero(float* p, uint64_t n) {
     // 16-byte stores over the aligned body, scalars at both ends
@@ -133,10 +133,13 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate(float* acc, uint64
 }
 
 // ---- tile bounds pre-pass ------------------------------------------------------
-// start[(b * ws + r) * (tiles + 1) + t] = first pair of rank r's bucket-b payload
-// whose index lies in tile t or later; start[..][tiles] = k.  One thread per pair:
-// pair p writes the entry of every tile that begins between pair p-1 and pair p
-// (usually none), so each entry is written exactly once for a sorted payload.
+// start[(b * (tiles + 1) + t) * ws + r] = first pair of rank r's bucket-b payload
+// whose index lies in tile t or later; entry t = tiles holds k.  The ws bounds of
+// a tile are adjacent, so a block of the accumulate kernel fetches its 2 * ws
+// bounds from one or two cache lines.  One thread per pair: pair p writes the
+// entry of every tile that begins between pair p-1 and pair p (usually none), so
+// each entry is written exactly once for a sorted payload.  The pair loads do not
+// wait for k: they stay inside the payload's stride and are masked afterwards.
 __global__ __launch_bounds__(kBlock) void k_sparse_bounds(WirePtrs wires, int ws, uint64_t wire_stride,
                                                           uint64_t n_total, uint64_t bucket_elems, uint32_t tiles,
                                                           uint32_t* start, int* status) {
@@ -145,25 +148,25 @@ __global__ __launch_bounds__(kBlock) void k_sparse_bounds(WirePtrs wires, int ws
     const uint64_t bn = (n_total - bstart) < bucket_elems ? (n_total - bstart) : bucket_elems;
     const uint32_t* wp = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride);
     const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
+    constexpr int PP = 4;  // pairs per thread, all loads issued before the first use
+    const uint32_t p0 = blockIdx.x * (kBlock * PP) + threadIdx.x;
+    uint32_t idx[PP], prev[PP];
+#pragma unroll
+    for (int j = 0; j < PP; j++) {
+        const uint32_t p = p0 + (uint32_t)j * kBlock;
+        const uint32_t pc = kmax == 0 ? 0 : (p < kmax ? p : kmax - 1);
+        idx[j] = kmax ? wp[1 + 2 * (uint64_t)pc] : 0u;
+        prev[j] = kmax ? wp[1 + 2 * (uint64_t)(pc > 0 ? pc - 1 : 0)] : 0u;
+    }
     uint32_t k = wp[0];
     if (k > kmax) {
         if (status) *status = MCCL_HIP_ERR_SIZE;
         k = 0;
     }
-    uint32_t* st = start + ((uint64_t)b * ws + r) * (tiles + 1);
-    constexpr int PP = 4;  // pairs per thread, all loads issued before the first use
-    const uint32_t p0 = blockIdx.x * (kBlock * PP) + threadIdx.x;
+    uint32_t* st = start + (uint64_t)b * (tiles + 1) * ws + r;  // entry of tile t at st[t * ws]
     if (k == 0) {
-        for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t <= tiles; t += gridDim.x * kBlock) st[t] = 0;
+        for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t <= tiles; t += gridDim.x * kBlock) st[(uint64_t)t * ws] = 0;
         return;
-    }
-    uint32_t idx[PP], prev[PP];
-#pragma unroll
-    for (int j = 0; j < PP; j++) {
-        const uint32_t p = p0 + (uint32_t)j * kBlock;
-        const uint32_t pc = p < k ? p : k - 1;
-        idx[j] = wp[1 + 2 * (uint64_t)pc];
-        prev[j] = wp[1 + 2 * (uint64_t)(pc > 0 ? pc - 1 : 0)];
     }
 #pragma unroll
     for (int j = 0; j < PP; j++) {
@@ -177,9 +180,9 @@ __global__ __launch_bounds__(kBlock) void k_sparse_bounds(WirePtrs wires, int ws
             if (prev[j] >= idx[j] && status) *status = MCCL_HIP_ERR_INDEX;  // not ascending
             t_prev = prev[j] / kAccTile;
         }
-        for (int64_t t = t_prev + 1; t <= (int64_t)t_hi; t++) st[t] = p;
+        for (int64_t t = t_prev + 1; t <= (int64_t)t_hi; t++) st[(uint64_t)t * ws] = p;
         if (p == k - 1)
-            for (uint32_t t = t_hi + 1; t <= tiles; t++) st[t] = k;
+            for (uint32_t t = t_hi + 1; t <= tiles; t++) st[(uint64_t)t * ws] = k;
     }
 }
 
@@ -202,7 +205,7 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint
     const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
     if (threadIdx.x < 2 * ws) {
         const int r = threadIdx.x < ws ? threadIdx.x : threadIdx.x - ws;
-        uint32_t v = start[((uint64_t)b * ws + r) * (tiles + 1) + t + (threadIdx.x < ws ? 0 : 1)];
+        uint32_t v = start[((uint64_t)b * (tiles + 1) + t + (threadIdx.x < ws ? 0 : 1)) * ws + r];
         if (v > kmax) v = kmax;  // stale bound of a malformed payload: stay inside the buffer
         if (threadIdx.x < ws) lo_s[r] = v; else hi_s[r] = v;
     }
