@@ -100,7 +100,10 @@ def main() -> int:
     roofline = {
         "bound": "hbm", "kernel": "k_ring_fold<f32,add>",
         "achieved": rate(fold_bytes, st["avg_ms"]), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": rate(fold_bytes, st["avg_ms"]) / HBM_PEAK_GBPS, "traffic": None,
+        "frac": rate(fold_bytes, st["avg_ms"]) / HBM_PEAK_GBPS,
+        # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded in
+        # profiles/ring_fold_f32_w8_96M_hbm_traffic.md (valid for the default workload only)
+        "traffic": 3_478_715_600 if N == N_GRAD else None,
         "bytes_per_launch": fold_bytes, "avg_launch_ms": st["avg_ms"], "min_launch_ms": st["min_ms"],
     }
 
