@@ -321,6 +321,10 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
 
 // ---- launch helpers -----------------------------------------------------------
 
+// One tile per block wherever possible: measured on MI355X, 16 K short-lived blocks
+// in address order stream faster (6.38 TB/s for the binary fold) than a persistent
+// grid of 2 K blocks striding through the array (6.20 TB/s).  The cap only bounds
+// the grid for very large arrays; the kernels stride when it applies.
 uint32_t stream_blocks(uint64_t work_tiles) {
     const uint64_t cap = (uint64_t)device_info().num_cus * (uint64_t)tuning().fold_blocks_per_cu;
     return clamp_u32(work_tiles, 1, cap);

@@ -19,7 +19,7 @@ struct DeviceInfo {
 const DeviceInfo& device_info();
 
 struct Tuning {
-    int fold_blocks_per_cu = 8;  // resident 256-thread blocks per CU for streaming kernels
+    int fold_blocks_per_cu = 256;  // grid cap of the streaming kernels, in blocks per CU
     int nontemporal = 1;         // 1: streaming loads/stores carry the `nt` hint (+8..12 % on MI355X)
     int topk_path = 0;           // 0 auto, 1 multi-pass exact path only, 2 single-pass path at any size
 };

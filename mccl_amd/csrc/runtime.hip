@@ -80,7 +80,7 @@ int mccl_hip_set_tuning(const char* key, int value) {
     if (!key) return MCCL_HIP_ERR_ARG;
     Tuning& t = tuning();
     if (!std::strcmp(key, "fold_blocks_per_cu")) {
-        if (value < 1 || value > 64) return MCCL_HIP_ERR_ARG;
+        if (value < 1 || value > 4096) return MCCL_HIP_ERR_ARG;
         t.fold_blocks_per_cu = value;
     } else if (!std::strcmp(key, "nontemporal")) {
         t.nontemporal = value ? 1 : 0;

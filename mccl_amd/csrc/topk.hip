@@ -18,9 +18,9 @@
 //   pass A     residual <- grad + residual in one streaming pass; elements with
 //              key >= lo ("candidates", about 1.7 k of them) are appended to
 //              per-bucket lists through per-wave LDS staging and counted in a
-//              2048-bin histogram that is linear in the key over [lo, hi)
+//              256-bin histogram that is linear in the key over [lo, hi)
 //   select1    finds the histogram bin that holds the k-th largest key and
-//              copies that bin's candidates (a handful) to a second list
+//              copies that bin's candidates (a few hundred) to a second list
 //   select2    one block per bucket: checks that the lists are complete and
 //              the threshold lies inside the window (else the bucket is handed
 //              to the exact fallback), finishes the radix select on the second
@@ -52,6 +52,10 @@ namespace {
 constexpr int kTile = 4096;    // exact path: elements per compaction tile
 constexpr int kBins0 = 2048;   // key[30:20]
 constexpr int kBinsR = 1024;   // key[19:10], key[9:0]
+#ifndef MCCLHIP_WINBINS
+#define MCCLHIP_WINBINS 256
+#endif
+constexpr int kWinBins = MCCLHIP_WINBINS;  // fast path: bins of the candidate window histogram
 constexpr int kHistWords = kBins0 + 2 * kBinsR;
 constexpr int kStateWords = 32;
 #ifndef MCCLHIP_ATILE
@@ -98,7 +102,7 @@ struct Geometry {
 struct Workspace {
     // zeroed at the start of every exact-path call; the single-pass path zeroes what it uses itself
     uint32_t* hist;         // [nbuckets][kHistWords]
-    uint32_t* hist_w;       // [nbuckets][kBins0]   candidates: window histogram, bin 2047 = above the window
+    uint32_t* hist_w;       // [nbuckets][kWinBins] candidates: window histogram, last bin = above the window
     uint32_t* state;        // [nbuckets][kStateWords]
     uint32_t* sub_count;    // [nbuckets][kNSub]
     uint32_t* etile_count;  // [nbuckets][etiles]
@@ -429,9 +433,9 @@ __global__ __launch_bounds__(kBlock) void k_topk_emit(float* residual, Geometry 
 // ================================= fast path ======================================
 
 // Window bin of a candidate key: linear in the key over [lo, hi), everything
-// at or above hi in bin kBins0 - 1.
+// at or above hi in bin kWinBins - 1.
 __device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32_t hi, uint32_t shift) {
-    return key >= hi ? (uint32_t)(kBins0 - 1) : (key - lo) >> shift;
+    return key >= hi ? (uint32_t)(kWinBins - 1) : (key - lo) >> shift;
 }
 
 // One block per bucket.  Loads kSample evenly spread elements of grad + residual
@@ -447,7 +451,7 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     __shared__ uint32_t scratch[kSelThreads / kWave + 2];
     const uint32_t b = blockIdx.x;
     // this bucket's accumulators for the kernels that follow start at zero
-    for (int i = threadIdx.x; i < kBins0; i += kSelThreads) w.hist_w[(uint64_t)b * kBins0 + i] = 0;
+    for (int i = threadIdx.x; i < kWinBins; i += kSelThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
     if (threadIdx.x < kNSub) w.sub_count[(uint64_t)b * kNSub + threadIdx.x] = 0;
     if (threadIdx.x < kStateWords) w.state[(uint64_t)b * kStateWords + threadIdx.x] = 0;
     const uint64_t bn = bucket_count(g, b);
@@ -516,7 +520,7 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
         uint32_t hi = active[0] ? prefix[0] : 0x7FFFFFFFu;
         if (hi < lo) hi = lo;
         uint32_t shift = 0;
-        while (((hi - lo) >> shift) >= (uint32_t)(kBins0 - 1)) shift++;
+        while (((hi - lo) >> shift) >= (uint32_t)(kWinBins - 1)) shift++;
         uint32_t* st = w.state + (uint64_t)b * kStateWords;
         st[S_LO_KEY] = lo;
         st[S_HI_KEY] = hi;
@@ -529,7 +533,7 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
 // One 8192-element tile per block, tiles in address order.
 __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __restrict__ grad, float* residual,
                                                              Geometry g, Workspace w) {
-    __shared__ uint32_t lh[kBins0];
+    __shared__ uint32_t lh[kWinBins];
     __shared__ uint32_t stage[kBlock / kWave][kStage][2];
     const uint32_t b = blockIdx.y, t = blockIdx.x;
     const uint64_t bn = bucket_count(g, b);
@@ -556,7 +560,9 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         }
     };
     issue(0);
-    for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
+#ifndef MCCLHIP_EXP_NOHIST
+    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
+#endif
     const uint32_t lo_key = w.state[(uint64_t)b * kStateWords + S_LO_KEY];
     const uint32_t hi_key = w.state[(uint64_t)b * kStateWords + S_HI_KEY];
     const uint32_t wshift = w.state[(uint64_t)b * kStateWords + S_SHIFT];
@@ -641,8 +647,10 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         }
     }
     if (staged) flush_stage();
+#ifndef MCCLHIP_EXP_NOHIST
     __syncthreads();
-    flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kBins0, kBins0);
+    flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kWinBins, kWinBins);
+#endif
 }
 
 // A block's view of up to 8 * kBlock consecutive (index, bits) entries: all
@@ -675,10 +683,10 @@ __global__ __launch_bounds__(kBlock) void k_topk_select1(Geometry g, Workspace w
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
     uint32_t need;
-    const uint32_t jstar = pick_bin<kBins0, kBlock>(w.hist_w + (uint64_t)b * kBins0, bucket_k(g, b), 0, &need, scratch);
+    const uint32_t jstar = pick_bin<kWinBins, kBlock>(w.hist_w + (uint64_t)b * kWinBins, bucket_k(g, b), 0, &need, scratch);
     if (s == 0 && threadIdx.x == 0) { st[S_P0] = jstar; st[S_R0] = need; }
     // fewer than k candidates, or the threshold lies above the window: fallback
-    if (jstar >= (uint32_t)(kBins0 - 1)) return;
+    if (jstar >= (uint32_t)(kWinBins - 1)) return;
     uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
     if (cnt > g.lsub) cnt = g.lsub;
     const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
@@ -764,7 +772,7 @@ __device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uin
 }
 
 // select, step 2: one block per bucket.  Validates the candidate lists, finishes
-// the radix select on list2 (keys of one window bin: 21 bits at most remain)
+// the radix select on list2 (keys of one window bin: 24 bits at most remain)
 // and resolves ties by index.
 __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, Geometry g, Workspace w,
                                                               uint8_t* wire, uint64_t wire_stride) {
@@ -778,17 +786,19 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     if (threadIdx.x < kNSub) over = w.sub_count[(uint64_t)b * kNSub + threadIdx.x] > g.lsub ? 1u : 0u;
     uint32_t any_over;
     block_exclusive_scan_n<kSelThreads>(over, scratch, &any_over);
-    if (any_over || jstar >= (uint32_t)(kBins0 - 1)) {
+    if (any_over || jstar >= (uint32_t)(kWinBins - 1)) {
         // incomplete candidate lists or threshold outside the window (rare): this block
         // runs the whole exact selection of the bucket; S_OK stays 0, so mark and emit skip it
+#ifndef MCCLHIP_EXP_NOFALLBACK
         bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
+#endif
         return;
     }
 
     const uint32_t* l2 = w.list2 + ((uint64_t)b * kNSub * g.lsub) * 2;
     const uint32_t count2 = st[S_N2];
     const uint32_t bin_lo = st[S_LO_KEY] + (jstar << st[S_SHIFT]);  // smallest key of the bin
-    uint32_t vprefix = 0;  // key - bin_lo: up to 21 bits, selected as 1 + 10 + 10
+    uint32_t vprefix = 0;  // key - bin_lo: up to 24 bits, selected as 4 + 10 + 10
     for (int r = 0; r < 3; r++) {
         const int shift = 20 - 10 * r;
         const int hs = shift + 10;
@@ -852,9 +862,14 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
 // list, zeroes the residual at the picks, and records (offset, count) per tile.
 // The emit kernel then only concatenates the runs.
 __global__ __launch_bounds__(kBlock) void k_topk_mark(float* residual, Geometry g, Workspace w) {
-    __shared__ uint32_t bm[kMarkTiles * (kETile / 32)];
-    __shared__ uint32_t pre[kMarkTiles * (kETile / 32)];  // picks of the tile before this word
-    __shared__ uint32_t tcount[kMarkTiles], toff[kMarkTiles];
+    // dynamic LDS, sized by the launch for ceil(etiles / kNSub) tiles (at most kMarkTiles):
+    // bitmap words, per-word pick prefix, per-tile count and offset
+    extern __shared__ uint32_t mark_lds[];
+    const uint32_t tmax = (g.etiles + kNSub - 1) / kNSub;
+    uint32_t* bm = mark_lds;
+    uint32_t* pre = bm + tmax * (kETile / 32);  // picks of the tile before this word
+    uint32_t* tcount = pre + tmax * (kETile / 32);
+    uint32_t* toff = tcount + tmax;
     const uint32_t b = blockIdx.y, s = blockIdx.x;
     const uint32_t* st = w.state + (uint64_t)b * kStateWords;
     if (!st[S_OK]) return;
@@ -947,7 +962,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_emit_fast(Geometry g, Workspace
 uint64_t align4(uint64_t words) { return (words + 3) & ~uint64_t(3); }
 
 uint64_t zeroed_words(const Geometry& g) {
-    return align4((uint64_t)g.nbuckets * kHistWords) + align4((uint64_t)g.nbuckets * kBins0) +
+    return align4((uint64_t)g.nbuckets * kHistWords) + align4((uint64_t)g.nbuckets * kWinBins) +
            align4((uint64_t)g.nbuckets * kStateWords) + align4((uint64_t)g.nbuckets * kNSub);
 }
 
@@ -961,7 +976,7 @@ Workspace carve(void* base, const Geometry& g) {
     Workspace w;
     uint32_t* p = (uint32_t*)base;
     w.hist = p;        p += align4((uint64_t)g.nbuckets * kHistWords);
-    w.hist_w = p;      p += align4((uint64_t)g.nbuckets * kBins0);
+    w.hist_w = p;      p += align4((uint64_t)g.nbuckets * kWinBins);
     w.state = p;       p += align4((uint64_t)g.nbuckets * kStateWords);
     w.sub_count = p;   p += align4((uint64_t)g.nbuckets * kNSub);
     w.etile_count = p; p += align4((uint64_t)g.nbuckets * g.etiles);
@@ -1052,7 +1067,9 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
         k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
         k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
-        k_topk_mark<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
+        const uint32_t tmax = (g.etiles + kNSub - 1) / kNSub;
+        const size_t mark_lds = (size_t)tmax * (2 * (kETile / 32) + 2) * sizeof(uint32_t);
+        k_topk_mark<<<dim3(kNSub, g.nbuckets), kBlock, mark_lds, st>>>(residual, g, w);
         k_topk_emit_fast<<<dim3((g.etiles + 3) / 4, g.nbuckets), kBlock, 0, st>>>(g, w, (uint8_t*)wire, wire_stride);
     } else {
         const uint64_t zw = zeroed_words(g);

@@ -44,7 +44,7 @@ def test_host_only_entry_points_agree_with_the_reference_formulas():
     assert lib.mccl_hip_topk_workspace_bytes(96_510_024, 6_553_600, 0.01) > 0
     assert lib.mccl_hip_set_tuning(b"fold_blocks_per_cu", 4) == 0
     assert lib.mccl_hip_get_tuning(b"fold_blocks_per_cu") == 4
-    assert lib.mccl_hip_set_tuning(b"fold_blocks_per_cu", 8) == 0
+    assert lib.mccl_hip_set_tuning(b"fold_blocks_per_cu", 256) == 0
     assert lib.mccl_hip_set_tuning(b"no_such_key", 1) == -6
 
 
