@@ -227,6 +227,17 @@ def main() -> int:
                                               "frac": rate(acc_bytes, sa["avg_ms"]) / HBM_PEAK_GBPS,
                                               "bytes": acc_bytes, "status": int(status)}
 
+    if a.only == "all":
+        # ---- FP16 compressor casts over the whole gradient (6 B / element each way) ----
+        half = torch.empty(N, dtype=torch.float16, device=dev)
+        c1 = stats(gpu_time(lambda: ops.cast_f32_to_f16(ranks[0], half))[1])
+        c2 = stats(gpu_time(lambda: ops.cast_f16_to_f32(half, out))[1])
+        extra["fp16_compress_cast"] = {"ms": c1["avg_ms"], "GBps": rate(6 * N, c1["avg_ms"]),
+                                       "frac": rate(6 * N, c1["avg_ms"]) / HBM_PEAK_GBPS}
+        extra["fp16_decompress_cast"] = {"ms": c2["avg_ms"], "GBps": rate(6 * N, c2["avg_ms"]),
+                                         "frac": rate(6 * N, c2["avg_ms"]) / HBM_PEAK_GBPS}
+        del half
+
     # ---- CPU baseline: the reference's CPU fold path restated, same workload ----
     cpu = None
     if not a.no_cpu:

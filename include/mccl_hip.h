@@ -190,6 +190,15 @@ int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_ele
  * every block, which costs about 3x the time on MI355X. */
 uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, int ws);
 
+/* ---- fp16 transport casts ------------------------------------------------ */
+
+/* FP16Compressor's casts (csrc/compression/FP16Compression.cpp:16-112):
+ * fp32 -> fp16 round-to-nearest-even with gradual underflow and overflow to
+ * infinity; NaN stays NaN (sign | 0x7C00 | mant >> 13 | 0x200); fp16 -> fp32
+ * exact.  dst holds n 16-bit / 32-bit elements. */
+int mccl_hip_cast_f32_to_f16(const float* src, void* dst, uint64_t n, void* stream);
+int mccl_hip_cast_f16_to_f32(const void* src, float* dst, uint64_t n, void* stream);
+
 /* ---- ordering ----------------------------------------------------------- */
 
 /* Replaces next_fence_event_value() + signal_mccl_fence_gpu()

@@ -51,7 +51,7 @@ def get_config() -> Optional[MCCLConfig]:
 def compressor_from_env():
     """The compressor the backend creates at start-up from MCCL_COMPRESSION /
     MCCL_TOPK_RATIO (csrc/backend/ProcessGroupMCCL.cpp:729-741): None for
-    "none", a device-resident TopKCompressor for "topk"."""
+    "none", a device-resident FP16Compressor for "fp16", TopKCompressor for "topk"."""
     import torch.distributed  # noqa: F401  (registers c10d base types for the extension)
     from mccl_amd import _C
 

@@ -22,7 +22,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmccl_hip.so")
 
-HIP_SOURCES = ["runtime.hip", "fold.hip", "topk.hip", "sparse.hip"]
+HIP_SOURCES = ["runtime.hip", "fold.hip", "topk.hip", "sparse.hip", "cast.hip"]
 
 # -ffp-contract=off: every fold is one IEEE operation per element, never an FMA.
 # packed-fp32-ops is switched off for all device code.
@@ -53,7 +53,7 @@ def build_lib(force: bool = True) -> str:
         o = os.path.join(OBJ, src.replace(".hip", ".o"))
         objs.append(o)
         jobs.append([hipcc, *HIPCC_FLAGS, "-c", s, "-o", o])
-    with cf.ThreadPoolExecutor(max_workers=4) as ex:
+    with cf.ThreadPoolExecutor(max_workers=5) as ex:
         list(ex.map(_run, jobs))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
     return LIB

@@ -3,7 +3,10 @@
 #include <c10/hip/HIPStream.h>
 
 #include "../../../include/mccl_hip.h"
+#include <hip/hip_runtime_api.h>
+
 #include "Errors.hpp"
+#include "FP16Compression.hpp"
 #include "HipKernels.hpp"
 #include "Logging.hpp"
 #include "TopKCompression.hpp"
@@ -13,10 +16,55 @@ namespace mccl {
 std::unique_ptr<Compressor> make_compressor(CompressionMode mode, double param) {
     switch (mode) {
         case CompressionMode::NONE: return nullptr;
+        case CompressionMode::FP16: return std::make_unique<FP16Compressor>();
         case CompressionMode::TOPK: return std::make_unique<TopKCompressor>(param > 0 ? param : 0.01);
         default:
             throw MCCLError("Unknown compression mode: " + std::to_string(static_cast<int>(mode)));
     }
+}
+
+namespace {
+void device_copy(void* dst, const void* src, size_t nbytes) {
+    if (nbytes == 0) return;
+    const hipError_t e = hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice,
+                                        c10::hip::getCurrentHIPStream().stream());
+    MCCL_CHECK(e == hipSuccess, std::string("FP16 passthrough copy failed: ") + hipGetErrorString(e));
+}
+}  // namespace
+
+// csrc/compression/FP16Compression.cpp:117-143
+size_t FP16Compressor::compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
+                                at::ScalarType dtype, uint64_t /*stable_id*/) {
+    if (dtype == at::kHalf) {
+        MCCL_CHECK(dst_capacity >= nbytes, "FP16 compress: buffer too small");
+        device_copy(dst, src, nbytes);
+        return nbytes;
+    }
+    MCCL_CHECK(dtype == at::kFloat, "FP16 compression only supports float32 input");
+    const size_t count = nbytes / sizeof(float);
+    const size_t compressed_bytes = count * sizeof(uint16_t);
+    MCCL_CHECK(dst_capacity >= compressed_bytes, "FP16 compress: buffer too small");
+    throw_on_status(mccl_hip_cast_f32_to_f16(static_cast<const float*>(src), dst, count,
+                                             c10::hip::getCurrentHIPStream().stream()),
+                    "FP16 compress");
+    MCCL_TRACE("FP16 compress: %zu -> %zu bytes", nbytes, compressed_bytes);
+    return compressed_bytes;
+}
+
+// csrc/compression/FP16Compression.cpp:145-163
+void FP16Compressor::decompress(const void* src, size_t compressed_size, void* dst, size_t nbytes,
+                                at::ScalarType dtype) {
+    if (dtype == at::kHalf) {
+        MCCL_CHECK(compressed_size == nbytes, "FP16 decompress: size mismatch");
+        device_copy(dst, src, nbytes);
+        return;
+    }
+    MCCL_CHECK(dtype == at::kFloat, "FP16 decompression only supports float32 output");
+    const size_t count = nbytes / sizeof(float);
+    MCCL_CHECK(compressed_size == count * sizeof(uint16_t), "FP16 decompress: compressed size mismatch");
+    throw_on_status(mccl_hip_cast_f16_to_f32(src, static_cast<float*>(dst), count,
+                                             c10::hip::getCurrentHIPStream().stream()),
+                    "FP16 decompress");
 }
 
 TopKCompressor::TopKCompressor(double k_ratio) : k_ratio_(k_ratio) {

@@ -37,9 +37,8 @@ public:
     virtual std::string name() const = 0;
 };
 
-/// NONE -> nullptr, TOPK -> TopKCompressor(param > 0 ? param : 0.01); FP16 is
-/// not part of this build and throws, like an unknown mode
-/// (csrc/compression/Compression.cpp:8-20).
+/// NONE -> nullptr, FP16 -> FP16Compressor, TOPK -> TopKCompressor(param > 0 ?
+/// param : 0.01); anything else throws (csrc/compression/Compression.cpp:8-20).
 std::unique_ptr<Compressor> make_compressor(CompressionMode mode, double param = 0.0);
 
 }  // namespace mccl

@@ -15,6 +15,7 @@
 #include "HipKernels.hpp"
 #include "Options.hpp"
 #include "TensorChecks.hpp"
+#include "FP16Compression.hpp"
 #include "TopKCompression.hpp"
 
 namespace py = pybind11;
@@ -162,9 +163,35 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             if (!t.defined()) return py::none();
             return py::cast(t);
         });
+    py::class_<mccl::FP16Compressor>(m, "FP16Compressor")
+        .def(py::init<>())
+        .def("name", &mccl::FP16Compressor::name)
+        .def("max_compressed_size", &mccl::FP16Compressor::max_compressed_size)
+        .def("compress", [](mccl::FP16Compressor& c, const at::Tensor& t, py::object capacity) {
+            mccl::check_single_tensor(t);
+            const size_t nbytes = mccl::tensor_nbytes(t);
+            const size_t cap = capacity.is_none() ? c.max_compressed_size(nbytes) : capacity.cast<size_t>();
+            at::Tensor out = at::empty({static_cast<int64_t>(cap)},
+                                       at::TensorOptions().dtype(at::kByte).device(t.device()));
+            const size_t used = c.compress(t.data_ptr(), nbytes, out.data_ptr(), cap, t.scalar_type());
+            return out.narrow(0, 0, static_cast<int64_t>(used));
+        }, py::arg("tensor"), py::arg("capacity") = py::none(),
+           "Half-precision payload of a float32 bucket (a float16 bucket is copied) as a uint8 device tensor")
+        .def("decompress", [](mccl::FP16Compressor& c, const at::Tensor& wire, int64_t numel, py::object size,
+                              at::ScalarType dtype) {
+            at::Tensor out = at::empty({numel}, at::TensorOptions().dtype(dtype).device(wire.device()));
+            const size_t sz = size.is_none() ? static_cast<size_t>(wire.numel()) : size.cast<size_t>();
+            c.decompress(wire.data_ptr(), sz, out.data_ptr(), static_cast<size_t>(numel) * out.element_size(), dtype);
+            return out;
+        }, py::arg("wire"), py::arg("numel"), py::arg("compressed_size") = py::none(),
+           py::arg("dtype") = at::kFloat);
     m.def("make_compressor", [](mccl::CompressionMode mode, double param) -> py::object {
         auto c = mccl::make_compressor(mode, param);
         if (!c) return py::none();
+        if (auto* half = dynamic_cast<mccl::FP16Compressor*>(c.get())) {
+            c.release();
+            return py::cast(half, py::return_value_policy::take_ownership);
+        }
         auto* topk = dynamic_cast<mccl::TopKCompressor*>(c.get());
         MCCL_CHECK(topk != nullptr, "unexpected compressor type");
         c.release();

@@ -174,6 +174,24 @@ def sparse_accumulate(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_str
     return acc
 
 
+def cast_f32_to_f16(src: torch.Tensor, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(src, "src")
+    if dst is None:
+        dst = torch.empty(src.numel(), dtype=torch.float16, device=src.device)
+    _lib.check(_lib.load().mccl_hip_cast_f32_to_f16(src.data_ptr(), dst.data_ptr(), src.numel(), _stream()),
+               "cast_f32_to_f16")
+    return dst
+
+
+def cast_f16_to_f32(src: torch.Tensor, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(src, "src")
+    if dst is None:
+        dst = torch.empty(src.numel(), dtype=torch.float32, device=src.device)
+    _lib.check(_lib.load().mccl_hip_cast_f16_to_f32(src.data_ptr(), dst.data_ptr(), src.numel(), _stream()),
+               "cast_f16_to_f32")
+    return dst
+
+
 def fence_signal() -> int:
     t = C.c_uint64(0)
     _lib.check(_lib.load().mccl_hip_fence_signal(_stream(), C.byref(t)), "fence_signal")

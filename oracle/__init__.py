@@ -44,6 +44,9 @@ def _load():
         "orc_bf16_to_f32": (f32, [C.c_uint16]),
         "orc_f32_to_bf16": (C.c_uint16, [f32]),
         "orc_convert": (i32, [vp, vp, i64, i32]),
+        "orc_f32_to_f16_transport": (C.c_uint16, [f32]),
+        "orc_fp16_compress": (i64, [vp, i64, vp, i64, i32]),
+        "orc_fp16_decompress": (i32, [vp, i64, vp, i64, i32]),
         "orc_fold2_f32": (i32, [vp, vp, i64, i32, i32]),
         "orc_scale_f32": (i32, [vp, i64, f32, i32]),
         "orc_fold2_scale_f32": (i32, [vp, vp, i64, f32, i32]),
@@ -104,6 +107,24 @@ def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
 
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     return _convert(x.astype(np.float32, copy=False), 3, np.uint16)
+
+
+# ---- FP16 compressor ----------------------------------------------------------
+def fp16_compress(data: np.ndarray, dtype: int = F32, capacity=None):
+    """Wire bytes (uint8 array), or the negative status."""
+    data = np.ascontiguousarray(data)
+    cap = data.nbytes if capacity is None else capacity
+    out = np.zeros(max(cap, 1), dtype=np.uint8)
+    rc = int(lib.orc_fp16_compress(_p(data), data.nbytes, _p(out), cap, dtype))
+    return rc if rc < 0 else out[:rc].copy()
+
+
+def fp16_decompress(wire: np.ndarray, count: int, dtype: int = F32, size=None):
+    """(dense array of `count` elements, status)."""
+    wire = np.ascontiguousarray(wire)
+    dst = np.zeros(count, dtype=np.float32 if dtype == F32 else np.uint16)
+    rc = int(lib.orc_fp16_decompress(_p(wire), wire.nbytes if size is None else size, _p(dst), dst.nbytes, dtype))
+    return dst, rc
 
 
 # ---- folds (in place on dst; dst is returned) -------------------------------
@@ -258,9 +279,9 @@ class RefCompressor:
         return out[:rc].copy()
 
     def decompress(self, wire: np.ndarray, count: int, size=None, dtype: int = F32):
-        dst = np.empty(count, dtype=np.float32)
+        dst = np.zeros(count, dtype=np.uint16 if dtype == F16 else np.float32)
         rc = self.l.ref_decompress(self.h, _p(wire), wire.size if size is None else size,
-                                   _p(dst), count * 4, dtype)
+                                   _p(dst), dst.nbytes, dtype)
         return dst, int(rc)
 
     def buffer_count(self) -> int:

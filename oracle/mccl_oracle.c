@@ -86,7 +86,46 @@ uint16_t orc_f32_to_bf16(float f) {
     return (uint16_t)((u + bias) >> 16);
 }
 
-/* Array forms: kind 0 f16->f32, 1 f32->f16, 2 bf16->f32, 3 f32->bf16. */
+/* csrc/compression/FP16Compression.cpp:47-51: a NaN keeps its sign and top
+ * mantissa bits and gets the quiet bit; everything else is plain RNE. */
+uint16_t orc_f32_to_f16_transport(float f) {
+    uint32_t x = f2u(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u)
+        return (uint16_t)(((x >> 16) & 0x8000u) | 0x7C00u | ((x & 0x7FFFFFu) >> 13) | 0x200u);
+    return orc_f32_to_f16(f);
+}
+
+/* csrc/compression/FP16Compression.cpp:117-143 */
+int64_t orc_fp16_compress(const void* src, int64_t nbytes, void* dst, int64_t capacity, int dtype) {
+    if (dtype == ORC_F16) {
+        if (capacity < nbytes) return ORC_ERR_CAPACITY;
+        memcpy(dst, src, (size_t)nbytes);
+        return nbytes;
+    }
+    if (dtype != ORC_F32) return ORC_ERR_DTYPE;
+    int64_t count = nbytes / 4;
+    if (capacity < count * 2) return ORC_ERR_CAPACITY;
+    for (int64_t i = 0; i < count; i++)
+        ((uint16_t*)dst)[i] = orc_f32_to_f16_transport(((const float*)src)[i]);
+    return count * 2;
+}
+
+/* csrc/compression/FP16Compression.cpp:145-163 */
+int orc_fp16_decompress(const void* src, int64_t compressed_size, void* dst, int64_t nbytes, int dtype) {
+    if (dtype == ORC_F16) {
+        if (compressed_size != nbytes) return ORC_ERR_SIZE;
+        memcpy(dst, src, (size_t)nbytes);
+        return ORC_OK;
+    }
+    if (dtype != ORC_F32) return ORC_ERR_DTYPE;
+    int64_t count = nbytes / 4;
+    if (compressed_size != count * 2) return ORC_ERR_SIZE;
+    for (int64_t i = 0; i < count; i++) ((float*)dst)[i] = orc_f16_to_f32(((const uint16_t*)src)[i]);
+    return ORC_OK;
+}
+
+/* Array forms: kind 0 f16->f32, 1 f32->f16, 2 bf16->f32, 3 f32->bf16,
+ * 4 f32->f16 with the FP16 compressor's NaN rule. */
 int orc_convert(void* dst, const void* src, int64_t n, int kind) {
     for (int64_t i = 0; i < n; i++) {
         switch (kind) {
@@ -94,6 +133,7 @@ int orc_convert(void* dst, const void* src, int64_t n, int kind) {
             case 1: ((uint16_t*)dst)[i] = orc_f32_to_f16(((const float*)src)[i]); break;
             case 2: ((float*)dst)[i] = orc_bf16_to_f32(((const uint16_t*)src)[i]); break;
             case 3: ((uint16_t*)dst)[i] = orc_f32_to_bf16(((const float*)src)[i]); break;
+            case 4: ((uint16_t*)dst)[i] = orc_f32_to_f16_transport(((const float*)src)[i]); break;
             default: return ORC_ERR_ARG;
         }
     }

@@ -60,8 +60,21 @@ float orc_f16_to_f32(uint16_t h);
 uint16_t orc_f32_to_f16(float f);
 float orc_bf16_to_f32(uint16_t b);
 uint16_t orc_f32_to_bf16(float f);
-/* Array forms: kind 0 f16->f32, 1 f32->f16, 2 bf16->f32, 3 f32->bf16. */
+/* Array forms: kind 0 f16->f32, 1 f32->f16, 2 bf16->f32, 3 f32->bf16,
+ * 4 f32->f16 with the FP16 compressor's NaN rule. */
 int orc_convert(void* dst, const void* src, int64_t n, int kind);
+
+/* ---- FP16 compressor (csrc/compression/FP16Compression.cpp:16-165) ----
+ * Follows the reference's target-platform (NEON) branch: IEEE RNE with
+ * gradual underflow; NaN -> sign | 0x7C00 | mant >> 13 | 0x200 (:47-51).
+ * The reference's portable branch differs only in flushing half subnormals
+ * to zero (:58-59, :102-103) and in leaving signalling NaNs unquieted when
+ * widening (:104-105).  dtype is ORC_F32 (cast) or ORC_F16 (passthrough).
+ * compress returns the byte count or ORC_ERR_CAPACITY / ORC_ERR_DTYPE;
+ * decompress returns ORC_OK or ORC_ERR_SIZE / ORC_ERR_DTYPE. */
+uint16_t orc_f32_to_f16_transport(float f);
+int64_t orc_fp16_compress(const void* src, int64_t nbytes, void* dst, int64_t capacity, int dtype);
+int orc_fp16_decompress(const void* src, int64_t compressed_size, void* dst, int64_t nbytes, int dtype);
 
 /* ---- binary folds, in place on dst; `threads` <= 0 picks the reference's
  *      job split (>= 1 Mi floats per job, at most 8 jobs). ---- */

@@ -39,8 +39,8 @@ def test_make_compressor_rules(C):
     c = C.make_compressor(C.CompressionMode.TOPK, 0.0)          # param <= 0 -> 0.01
     assert c.name() == "topk" and c.max_compressed_size(6_553_600 * 4) == 4 + 8 * 65_537
     assert C.make_compressor(C.CompressionMode.TOPK, 0.1).max_compressed_size(4000) == 4 + 8 * 101
-    with pytest.raises(RuntimeError, match="Unknown compression mode"):
-        C.make_compressor(C.CompressionMode.FP16, 0.0)
+    h = C.make_compressor(C.CompressionMode.FP16, 0.0)          # FP16Compression.cpp:165-168
+    assert isinstance(h, C.FP16Compressor) and h.name() == "fp16" and h.max_compressed_size(4096) == 4096
     for bad in (0.0, -1.0, 1.5):
         with pytest.raises(RuntimeError, match=r"k_ratio must be in \(0, 1\]"):
             C.TopKCompressor(bad)
