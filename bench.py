@@ -288,6 +288,18 @@ def main() -> int:
                 "cores": 1, "kind": "reference",
                 "sample": f"one 25 MiB bucket, {reps} repetitions of the reference's compiled TopKCompressor::compress"}
 
+    if a.only == "all":
+        # ---- step-wise ring driver: 8 ranks, chunked ring allreduce (reduce-scatter folds,
+        # all-gather copies, AVG scale on every rank), one HIP stream per rank with fences.
+        # Runs last: it reduces `ranks` in place.
+        import torch.distributed  # noqa: F401
+        from mccl_amd import _C
+        group = _C.LoopbackGroup(W)
+        rd = stats(gpu_time(lambda: group.allreduce_ring(ranks, ops.AVG, True), steps=max(3, K // 4), warmup=1)[1])
+        rd_bytes = ((W - 1) * 12 + (W - 1) * 8 + W * 8) * N
+        extra["ring_driver_allreduce_w8"] = {"ms": rd["avg_ms"], "GBps": rate(rd_bytes, rd["avg_ms"]),
+                                             "bytes": rd_bytes, "launches": 2 * W * 2 * (W - 1) + W}
+
     line = {
         "metric": "HBM GB/s (% of peak) for fp32 bucket fold and top-k 1% compress, 1 GPU",
         "value": fold_gbps, "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": WU,

@@ -14,6 +14,7 @@
 #include "Errors.hpp"
 #include "HipKernels.hpp"
 #include "Options.hpp"
+#include "RingDriver.hpp"
 #include "TensorChecks.hpp"
 #include "FP16Compression.hpp"
 #include "TopKCompression.hpp"
@@ -134,7 +135,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     });
 
     // ---- compressor -------------------------------------------------------------
-    py::class_<mccl::TopKCompressor>(m, "TopKCompressor")
+    py::class_<mccl::Compressor>(m, "Compressor");
+    py::class_<mccl::TopKCompressor, mccl::Compressor>(m, "TopKCompressor")
         .def(py::init<double>(), py::arg("k_ratio"))
         .def("name", &mccl::TopKCompressor::name)
         .def("max_compressed_size", &mccl::TopKCompressor::max_compressed_size)
@@ -163,7 +165,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             if (!t.defined()) return py::none();
             return py::cast(t);
         });
-    py::class_<mccl::FP16Compressor>(m, "FP16Compressor")
+    py::class_<mccl::FP16Compressor, mccl::Compressor>(m, "FP16Compressor")
         .def(py::init<>())
         .def("name", &mccl::FP16Compressor::name)
         .def("max_compressed_size", &mccl::FP16Compressor::max_compressed_size)
@@ -198,4 +200,69 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return py::cast(topk, py::return_value_policy::take_ownership);
     }, py::arg("mode"), py::arg("param") = 0.0);
     m.def("_compression_stable_id", &stable_id_of);
+
+    // ---- ring plan, payload framing, W ranks on one GPU ------------------------
+    m.def("_ring_plan", [](int rank, int ws, bool chunked) {
+        py::list out;
+        for (const auto& st : mccl::ring_plan(rank, ws, chunked ? mccl::RingAlgo::CHUNKED : mccl::RingAlgo::BASIC))
+            out.append(py::make_tuple(st.send_idx, st.recv_idx, st.send_tid, st.recv_tid,
+                                      st.kind == mccl::RingRecvKind::REDUCE ? "reduce" : "copy"));
+        return out;
+    }, py::arg("rank"), py::arg("world_size"), py::arg("chunked") = true,
+       "(send_idx, recv_idx, send_tid, recv_tid, kind) per step: reduce-scatter, then all-gather");
+    m.def("_ring_chunk_views", [](const at::Tensor& t, int ws, bool chunked) {
+        return mccl::ring_chunk_views(t, ws, chunked ? mccl::RingAlgo::CHUNKED : mccl::RingAlgo::BASIC);
+    }, py::arg("tensor"), py::arg("world_size"), py::arg("chunked") = true);
+    m.def("_ring_algo_from_env", [] { return mccl::ring_algo_from_env() == mccl::RingAlgo::CHUNKED ? "chunked" : "basic"; });
+    m.def("_compressed_pack", [](mccl::Compressor& c, const at::Tensor& t) {
+        mccl::CompressedFrame f = mccl::compressed_pack(&c, t);
+        return py::make_tuple(f.wire_size, f.payload);
+    }, py::arg("compressor"), py::arg("tensor"), "(size header, payload of exactly that many bytes)");
+    m.def("_compressed_unpack", [](mccl::Compressor& c, uint32_t wire_size, const at::Tensor& payload, at::Tensor out) {
+        mccl::CompressedFrame f;
+        f.wire_size = wire_size;
+        f.payload = payload;
+        mccl::compressed_unpack(&c, f, out);
+        return out;
+    }, py::arg("compressor"), py::arg("wire_size"), py::arg("payload"), py::arg("out"));
+
+    py::class_<mccl::LoopbackGroup>(m, "LoopbackGroup")
+        .def(py::init([](int ws, py::object opts, bool rank_streams) {
+            if (opts.is_none()) return std::make_unique<mccl::LoopbackGroup>(ws, mccl::MCCLOptions(), rank_streams);
+            return std::make_unique<mccl::LoopbackGroup>(ws, *opts.cast<c10::intrusive_ptr<mccl::MCCLOptions>>(),
+                                                         rank_streams);
+        }), py::arg("world_size"), py::arg("options") = py::none(), py::arg("rank_streams") = true)
+        .def("size", &mccl::LoopbackGroup::size)
+        .def("compressor", [](mccl::LoopbackGroup& g, int rank) -> mccl::Compressor* {
+            MCCL_CHECK(rank >= 0 && rank < g.size(), "rank out of range");
+            return g.compressor(rank);
+        }, py::return_value_policy::reference_internal)
+        .def("allreduce", [](mccl::LoopbackGroup& g, std::vector<at::Tensor> t, int op) {
+            g.allreduce(t, static_cast<c10d::ReduceOp::RedOpType>(op));
+        }, py::arg("rank_tensors"), py::arg("op") = 0)
+        .def("allreduce_coalesced", [](mccl::LoopbackGroup& g, std::vector<std::vector<at::Tensor>> lists, int op) {
+            g.allreduce_coalesced(lists, static_cast<c10d::ReduceOp::RedOpType>(op));
+        }, py::arg("rank_lists"), py::arg("op") = 0)
+        .def("allreduce_ring", [](mccl::LoopbackGroup& g, std::vector<at::Tensor> t, int op, bool chunked) {
+            g.allreduce_ring(t, static_cast<c10d::ReduceOp::RedOpType>(op),
+                             chunked ? mccl::RingAlgo::CHUNKED : mccl::RingAlgo::BASIC);
+        }, py::arg("rank_tensors"), py::arg("op") = 0, py::arg("chunked") = true)
+        .def("allreduce_two_rank", [](mccl::LoopbackGroup& g, std::vector<at::Tensor> t, int op) {
+            g.allreduce_two_rank(t, static_cast<c10d::ReduceOp::RedOpType>(op));
+        }, py::arg("rank_tensors"), py::arg("op") = 0)
+        .def("allreduce_small", [](mccl::LoopbackGroup& g, std::vector<at::Tensor> t, int op) {
+            g.allreduce_small(t, static_cast<c10d::ReduceOp::RedOpType>(op));
+        }, py::arg("rank_tensors"), py::arg("op") = 0)
+        .def("stats", [](const mccl::LoopbackGroup& g) {
+            const auto& s = g.stats();
+            py::dict d;
+            d["collectives"] = s.collectives;
+            d["reduce_launches"] = s.reduce_launches;
+            d["copy_launches"] = s.copy_launches;
+            d["fences_signalled"] = s.fences_signalled;
+            d["stream_waits"] = s.stream_waits;
+            d["wire_bytes"] = s.wire_bytes;
+            d["last_algo"] = s.last_algo;
+            return d;
+        });
 }

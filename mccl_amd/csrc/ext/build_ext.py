@@ -10,7 +10,7 @@ import sysconfig
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(os.path.dirname(HERE))
 OBJ = os.path.join(PKG, "build", "ext")
-SOURCES = ["HipKernels.cpp", "Compression.cpp", "Registration.cpp"]
+SOURCES = ["HipKernels.cpp", "Compression.cpp", "RingDriver.cpp", "Registration.cpp"]
 
 
 def target() -> str:
@@ -42,7 +42,7 @@ def build(force: bool = True) -> str:
         o = os.path.join(OBJ, s.replace(".cpp", ".o"))
         objs.append(o)
         jobs.append([cxx, *flags, *inc, "-c", os.path.join(HERE, s), "-o", o])
-    with cf.ThreadPoolExecutor(max_workers=3) as ex:
+    with cf.ThreadPoolExecutor(max_workers=4) as ex:
         list(ex.map(_run, jobs))
     out = target()
     _run([cxx, "-shared", "-o", out, *objs, f"-L{PKG}", "-lmccl_hip", f"-L{tdir}/lib", "-lc10", "-lc10_hip",
