@@ -52,19 +52,10 @@ namespace {
 constexpr int kTile = 4096;    // exact path: elements per compaction tile
 constexpr int kBins0 = 2048;   // key[30:20]
 constexpr int kBinsR = 1024;   // key[19:10], key[9:0]
-#ifndef MCCLHIP_WINBINS
-#define MCCLHIP_WINBINS 256
-#endif
-constexpr int kWinBins = MCCLHIP_WINBINS;  // fast path: bins of the candidate window histogram
+constexpr int kWinBins = 256;  // fast path: bins of the candidate window histogram
 constexpr int kHistWords = kBins0 + 2 * kBinsR;
 constexpr int kStateWords = 32;
-#ifndef MCCLHIP_ATILE
-#define MCCLHIP_ATILE 8192
-#endif
-#ifndef MCCLHIP_AUNROLL
-#define MCCLHIP_AUNROLL 2
-#endif
-constexpr int kATile = MCCLHIP_ATILE;   // fast path: elements per pass-A block
+constexpr int kATile = 8192;   // fast path: elements per pass-A block
 constexpr int kETile = 8192;   // fast path: elements per emission block (256 bitmap words, one per thread)
 static_assert(kATile == kETile, "a candidate sub-list must hold whole emission tiles");
 constexpr int kNSub = 64;      // fast path: candidate sub-lists per bucket
@@ -528,12 +519,14 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     }
 }
 
-// residual <- grad + residual; candidates (key >= lo) are counted in the window
-// histogram and appended to the bucket's sub-list (tile number mod kNSub).
-// One 8192-element tile per block, tiles in address order.
+// residual <- grad + residual; candidates (key >= lo) are appended to the
+// bucket's sub-list (tile number mod kNSub).  One 8192-element tile per block,
+// tiles in address order.  Nothing else happens here: the window histogram is
+// built afterwards from the lists (k_topk_window_hist), because flushing a
+// per-block histogram with device-scope atomics from every one of the 12,000
+// streaming blocks cost 15 % of this kernel's time.
 __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __restrict__ grad, float* residual,
                                                              Geometry g, Workspace w) {
-    __shared__ uint32_t lh[kWinBins];
     __shared__ uint32_t stage[kBlock / kWave][kStage][2];
     const uint32_t b = blockIdx.y, t = blockIdx.x;
     const uint64_t bn = bucket_count(g, b);
@@ -541,13 +534,12 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
     if (e0 >= bn) return;
     const float* gp = grad + (uint64_t)b * g.bucket_elems;
     float* rp = residual + (uint64_t)b * g.bucket_elems;
-    constexpr int U = MCCLHIP_AUNROLL;
+    constexpr int U = 2;
     constexpr int ROUNDS = kATile / (kBlock * 4 * U);
     const uint64_t tile_end = (e0 + kATile) < bn ? (e0 + kATile) : bn;
     const uint64_t nfull = (tile_end - e0) / 4;  // full vectors in this tile
     // The streaming loads of a round are issued one round ahead: round 0's before
-    // the block's set-up (LDS clear, bucket parameters), round r+1's before round r
-    // is processed, so the set-up latencies hide behind the HBM latency.
+    // the bucket parameters are read, round r+1's before round r is processed.
     u4a gv[ROUNDS][U], rv[ROUNDS][U];
     auto issue = [&](int round) {
 #pragma unroll
@@ -560,13 +552,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         }
     };
     issue(0);
-#ifndef MCCLHIP_EXP_NOHIST
-    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
-#endif
     const uint32_t lo_key = w.state[(uint64_t)b * kStateWords + S_LO_KEY];
-    const uint32_t hi_key = w.state[(uint64_t)b * kStateWords + S_HI_KEY];
-    const uint32_t wshift = w.state[(uint64_t)b * kStateWords + S_SHIFT];
-    __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const uint32_t sub = t % kNSub;
@@ -595,31 +581,32 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         for (int u = 0; u < U; u++) {
             const uint64_t vi = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
             u4a a = {0u, 0u, 0u, 0u};
-            bool cand[4] = {false, false, false, false};
-            const bool live = vi < nfull;
-            if (live) {
+            uint32_t mask4 = 0;  // which of this lane's four elements are candidates
+            if (vi < nfull) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const float adj = u2f(gv[round][u][q]) + u2f(rv[round][u][q]);
                     a[q] = f2u(adj);
-                    cand[q] = key_of(adj) >= lo_key;
+                    mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
                 }
                 __builtin_nontemporal_store(a, (u4u4*)(rp + e0 + vi * 4));
             }
-            const bool any = cand[0] | cand[1] | cand[2] | cand[3];
-            if (__ballot(any)) {  // wave-uniform
-                if (staged + 4 * kWave > kStage) flush_stage();
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const uint64_t m = __ballot(cand[q]);
-                    if (cand[q]) {
-                        const uint32_t pos = staged + __popcll(m & ((1ull << lane) - 1ull));
-                        stage[wave][pos][0] = (uint32_t)(e0 + vi * 4 + q);
-                        stage[wave][pos][1] = a[q];
-                        atomicAdd(&lh[window_bin(a[q] & 0x7FFFFFFFu, lo_key, hi_key, wshift)], 1u);
-                    }
-                    staged += (uint32_t)__popcll(m);
+            // One staging step per level: every lane that still holds a candidate stages its
+            // lowest one.  About 6 % of the lanes hold one, hardly any holds two, so the
+            // second trip is rare; per-element ballots would run four times on every vector.
+            uint64_t act = __ballot(mask4 != 0);
+            while (act) {  // wave-uniform
+                if (staged + kWave > kStage) flush_stage();
+                if (mask4) {
+                    const uint32_t q = (uint32_t)__ffs((int)mask4) - 1u;
+                    const uint32_t val = q == 0 ? a[0] : (q == 1 ? a[1] : (q == 2 ? a[2] : a[3]));
+                    const uint32_t pos = staged + __popcll(act & ((1ull << lane) - 1ull));
+                    stage[wave][pos][0] = (uint32_t)(e0 + vi * 4) + q;
+                    stage[wave][pos][1] = val;
+                    mask4 &= mask4 - 1u;
                 }
+                staged += (uint32_t)__popcll(act);
+                act = __ballot(mask4 != 0);
             }
         }
     }
@@ -641,16 +628,11 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
                 const uint32_t pos = staged + __popcll(m & ((1ull << lane) - 1ull));
                 stage[wave][pos][0] = (uint32_t)i;
                 stage[wave][pos][1] = bitsv;
-                atomicAdd(&lh[window_bin(bitsv & 0x7FFFFFFFu, lo_key, hi_key, wshift)], 1u);
             }
             staged += (uint32_t)__popcll(m);
         }
     }
     if (staged) flush_stage();
-#ifndef MCCLHIP_EXP_NOHIST
-    __syncthreads();
-    flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kWinBins, kWinBins);
-#endif
 }
 
 // A block's view of up to 8 * kBlock consecutive (index, bits) entries: all
@@ -670,6 +652,28 @@ __device__ __forceinline__ EntryChunk load_entries(const uint32_t* l, uint32_t b
         c.bits[j] = l[2 * (uint64_t)ii + 1];
     }
     return c;
+}
+
+// Window histogram of a bucket's candidates: one block per sub-list, counts in
+// LDS, one flush per block.
+__global__ __launch_bounds__(kBlock) void k_topk_window_hist(Geometry g, Workspace w) {
+    __shared__ uint32_t lh[kWinBins];
+    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
+    uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
+    if (cnt > g.lsub) cnt = g.lsub;
+    const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
+    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
+    __syncthreads();
+    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
+        const EntryChunk c = load_entries(l, base, cnt);
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (c.valid[j]) atomicAdd(&lh[window_bin(c.bits[j] & 0x7FFFFFFFu, lo, hi, shift)], 1u);
+    }
+    __syncthreads();
+    flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kWinBins, kWinBins);
 }
 
 // select, step 1: one block per candidate sub-list.  Finds the window bin that
@@ -789,9 +793,7 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     if (any_over || jstar >= (uint32_t)(kWinBins - 1)) {
         // incomplete candidate lists or threshold outside the window (rare): this block
         // runs the whole exact selection of the bucket; S_OK stays 0, so mark and emit skip it
-#ifndef MCCLHIP_EXP_NOFALLBACK
         bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
-#endif
         return;
     }
 
@@ -1065,6 +1067,7 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
         k_topk_sample<<<g.nbuckets, kSelThreads, 0, st>>>(grad, residual, g, w);
         const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
+        k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
         k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
         k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
         const uint32_t tmax = (g.etiles + kNSub - 1) / kNSub;
