@@ -49,8 +49,6 @@ __global__ __launch_bounds__(kBlock) void k_cast_f32_f16(const float* __restrict
 // store covers 1 KiB of consecutive addresses; kWidenQuads such groups per lane,
 // a block apart, keep several loads in flight.
 constexpr int kWidenQuads = 4;
-typedef uint32_t u2u2 __attribute__((ext_vector_type(2), aligned(2)));
-typedef uint32_t u2a __attribute__((ext_vector_type(2)));
 
 __global__ __launch_bounds__(kBlock) void k_cast_f16_f32(const uint16_t* __restrict__ src, float* __restrict__ dst,
                                                          uint64_t n) {

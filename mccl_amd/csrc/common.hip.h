@@ -18,6 +18,9 @@ constexpr int kWave = 64;
 typedef uint32_t u4a __attribute__((ext_vector_type(4)));
 typedef uint32_t u4u4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u4u2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t u2a __attribute__((ext_vector_type(2)));
+typedef uint32_t u2a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t u2u2 __attribute__((ext_vector_type(2), aligned(2)));
 typedef uint32_t u4u1 __attribute__((ext_vector_type(4), aligned(1)));
 
 enum { kAdd = 0, kMul = 1, kMin = 2, kMax = 3 };

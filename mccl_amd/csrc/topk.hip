@@ -56,13 +56,14 @@ constexpr int kWinBins = 256;  // fast path: bins of the candidate window histog
 constexpr int kHistWords = kBins0 + 2 * kBinsR;
 constexpr int kStateWords = 32;
 constexpr int kATile = 8192;   // fast path: elements per pass-A block
-constexpr int kETile = 8192;   // fast path: elements per emission block (256 bitmap words, one per thread)
-static_assert(kATile == kETile, "a candidate sub-list must hold whole emission tiles");
-constexpr int kNSub = 64;      // fast path: candidate sub-lists per bucket
-constexpr int kStage = 384;    // fast path: staged candidates per wavefront (>= 256: one vector's worth)
+constexpr int kRegion = 2048;  // fast path: elements per candidate region (one wavefront of a pass-A block)
+constexpr int kRegSlots = 64;  // fast path: candidate slots per region, one per lane of the wavefront that reads it
+static_assert(kATile == kRegion * (kBlock / kWave), "one region per wavefront");
+static_assert(kRegSlots == kWave, "a wavefront reads a region's slots in one go");
+constexpr uint32_t kDense = 0xFFFFFFFFu;  // region count: more candidates than slots, read the residual range itself
+constexpr int kNSub = 64;      // fast path: blocks per bucket in the kernels that walk the regions
 constexpr int kSelThreads = 1024;
 constexpr uint64_t kFastMinBucket = 1u << 18;
-constexpr int kMarkTiles = 24;  // fast path: emission tiles one mark block can hold in LDS
 constexpr int kSample = 12288;  // fast path: sampled elements per bucket (12 per select thread)
 
 // per-bucket state words
@@ -76,7 +77,8 @@ enum {
     S_OK = 7,             // fast path: 1 when select succeeded for this bucket
     S_ISTAR = 8,          // fast path: ties are taken while index <= this
     S_EXACT_HIST = 9,     // 1 when hist round 0 holds the full histogram
-    S_N2 = 10             // fast path: entries in list2
+    S_N2 = 10,            // fast path: entries in list2
+    S_THAT = 13           // fast path: predicted threshold key; pass A stores 0 for keys >= this
 };
 
 struct Geometry {
@@ -86,8 +88,8 @@ struct Geometry {
     uint32_t tiles;    // exact-path tiles per (full) bucket
     uint32_t k_full;   // k of a bucket with bucket_elems elements
     uint32_t k_last;   // k of the last bucket
-    uint32_t etiles;   // emission tiles per bucket
-    uint32_t lsub;     // capacity of one candidate sub-list (entries)
+    uint32_t regions;  // fast path: candidate regions allotted per bucket
+    uint32_t lcap2;    // fast path: capacity of a bucket's list2 (entries)
 };
 
 struct Workspace {
@@ -95,14 +97,14 @@ struct Workspace {
     uint32_t* hist;         // [nbuckets][kHistWords]
     uint32_t* hist_w;       // [nbuckets][kWinBins] candidates: window histogram, last bin = above the window
     uint32_t* state;        // [nbuckets][kStateWords]
-    uint32_t* sub_count;    // [nbuckets][kNSub]
-    uint32_t* etile_count;  // [nbuckets][etiles]
-    uint32_t* etile_off;    // [nbuckets][etiles]  start of the tile's run inside its sub-list's staging
     // scratch, written before read
     uint32_t* tile_gt;      // [nbuckets][tiles]
     uint32_t* tile_eq;      // [nbuckets][tiles]
-    uint32_t* list;         // [nbuckets][kNSub][lsub][2]  (index, bits)
-    uint32_t* list2;        // [nbuckets][kNSub * lsub][2] candidates of the threshold bin, later the staged picks
+    uint32_t* reg_cnt;      // [nbuckets][regions] candidates in the region's slots, or kDense
+    uint32_t* reg_pick;     // [nbuckets][regions] picks in the region
+    uint32_t* reg_off;      // [nbuckets][regions] picks in all regions before it
+    uint32_t* list;         // [nbuckets][regions][kRegSlots][2]  (index, bits), index order
+    uint32_t* list2;        // [nbuckets][lcap2][2] candidates of the threshold bin (index, key)
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -438,12 +440,11 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
                                                              const float* __restrict__ residual, Geometry g,
                                                              Workspace w) {
     __shared__ uint32_t keys[kSample];
-    __shared__ uint32_t lh[2][kBinsR];
+    __shared__ uint32_t lh[3][kBinsR];
     __shared__ uint32_t scratch[kSelThreads / kWave + 2];
     const uint32_t b = blockIdx.x;
     // this bucket's accumulators for the kernels that follow start at zero
     for (int i = threadIdx.x; i < kWinBins; i += kSelThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
-    if (threadIdx.x < kNSub) w.sub_count[(uint64_t)b * kNSub + threadIdx.x] = 0;
     if (threadIdx.x < kStateWords) w.state[(uint64_t)b * kStateWords + threadIdx.x] = 0;
     const uint64_t bn = bucket_count(g, b);
     const float* gp = grad + (uint64_t)b * g.bucket_elems;
@@ -471,17 +472,20 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     const uint32_t S = nsv * 4;
     const float ks = (float)bucket_k(g, b) * (float)S / (float)bn;
     const float margin = 6.0f * sqrtf(ks) + 16.0f;
-    uint32_t rank[2];
+    // ranks: 0 upper end of the window, 1 lower end, 2 the predicted threshold itself
+    constexpr int NR = 3;
+    uint32_t rank[NR];
     rank[0] = ks - margin >= 1.0f ? (uint32_t)(ks - margin) : 0u;  // 0: no upper end
     rank[1] = (uint32_t)(ks + margin) + 1u;                       // > S: no lower end
-    uint32_t prefix[2] = {0u, 0u}, want[2] = {rank[0], rank[1]};
-    const bool active[2] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S};
+    rank[2] = ks >= 1.0f ? (uint32_t)ks : 1u;
+    uint32_t prefix[NR] = {0u, 0u, 0u}, want[NR] = {rank[0], rank[1], rank[2]};
+    const bool active[NR] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S, rank[2] <= S};
     const int shifts[3] = {20, 10, 0};
     __syncthreads();
     for (int r = 0; r < 3; r++) {
-        // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves both ranks
+        // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves all ranks
         uint32_t* h0 = &lh[0][0];
-        for (int i = threadIdx.x; i < 2 * kBinsR; i += kSelThreads) h0[i] = 0;
+        for (int i = threadIdx.x; i < NR * kBinsR; i += kSelThreads) h0[i] = 0;
         __syncthreads();
         const int shift = shifts[r];
         for (uint32_t i = threadIdx.x; i < S; i += kSelThreads) {
@@ -491,13 +495,13 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
             } else {
                 const int hs = shift + 10;
 #pragma unroll
-                for (int z = 0; z < 2; z++)
+                for (int z = 0; z < NR; z++)
                     if (active[z] && (key >> hs) == (prefix[z] >> hs)) atomicAdd(&lh[z][(key >> shift) & (kBinsR - 1)], 1u);
             }
         }
         __syncthreads();
 #pragma unroll
-        for (int z = 0; z < 2; z++) {
+        for (int z = 0; z < NR; z++) {
             if (!active[z]) continue;
             uint32_t left, bin;
             if (r == 0) bin = pick_bin<kBins0, kSelThreads>(h0, want[z], 0, &left, scratch);
@@ -516,62 +520,191 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
         st[S_LO_KEY] = lo;
         st[S_HI_KEY] = hi;
         st[S_SHIFT] = shift;
+        // never below lo: every pre-zeroed element must be a listed candidate
+        uint32_t that = active[2] ? prefix[2] : 0x7FFFFFFFu;
+        st[S_THAT] = that < lo ? lo : that;
     }
 }
 
-// residual <- grad + residual; candidates (key >= lo) are appended to the
-// bucket's sub-list (tile number mod kNSub).  One 8192-element tile per block,
-// tiles in address order.  Nothing else happens here: the window histogram is
-// built afterwards from the lists (k_topk_window_hist), because flushing a
-// per-block histogram with device-scope atomics from every one of the 12,000
-// streaming blocks cost 15 % of this kernel's time.
+// ---- candidate regions ------------------------------------------------------------
+// A region is the kRegion consecutive elements one wavefront of a pass-A block
+// streams.  Its candidates land, in index order, in the region's kRegSlots slots
+// of `list` (slot = lane of the wave that later reads it) and their number in
+// reg_cnt.  A region with more candidates than slots is marked kDense: readers
+// then take every element of the region's residual range as a candidate.  No
+// atomics and no shared capacity are involved, so nothing can overflow.
+
+// One chunk of a block's slot range: kChunk slots per thread, all loads issued
+// before the first use.  A wavefront's 64 lanes cover exactly one region per j.
+constexpr int kChunk = 8;
+struct SlotChunk {
+    uint32_t idx[kChunk], bits[kChunk], region[kChunk];
+    bool valid[kChunk];   // the slot holds a candidate
+    uint32_t dense_mask;  // bit j: the region of slot j is dense
+};
+__device__ __forceinline__ SlotChunk load_slots(const uint32_t* reg_cnt_b, const uint32_t* list_b, uint32_t slot0,
+                                                uint32_t slot_end) {
+    SlotChunk c;
+    uint32_t cnt[kChunk];
+    c.dense_mask = 0;
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) {
+        const uint32_t slot = slot0 + (uint32_t)j * kBlock + threadIdx.x;
+        c.region[j] = slot / kRegSlots;
+        cnt[j] = slot < slot_end ? reg_cnt_b[c.region[j]] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) {
+        const uint32_t slot = slot0 + (uint32_t)j * kBlock + threadIdx.x;
+        c.dense_mask |= (cnt[j] == kDense ? 1u : 0u) << j;
+        c.valid[j] = cnt[j] != kDense && (slot % kRegSlots) < cnt[j];
+        u2a e = {0u, 0u};
+        if (c.valid[j]) e = *(const u2a*)(list_b + 2 * (uint64_t)slot);
+        c.idx[j] = e[0];
+        c.bits[j] = e[1];
+    }
+    return c;
+}
+
+// Dense regions met by a block are noted in LDS while it walks its slots (one
+// lane per region notes it), so the rare dense work is a loop over that short
+// list.  dl[0] counts, dl[1..kDenseList] hold region numbers; when more dense
+// regions turn up than fit, the caller walks all its regions instead.
+constexpr uint32_t kDenseList = 62;
+__device__ __forceinline__ void note_dense(const SlotChunk& c, uint32_t* dl) {
+    if (c.dense_mask && (threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+        for (int j = 0; j < kChunk; j++) {
+            if ((c.dense_mask >> j) & 1u) {
+                const uint32_t p = atomicAdd(&dl[0], 1u);
+                if (p < kDenseList) dl[1 + p] = c.region[j];
+            }
+        }
+    }
+}
+// The i-th dense region a wavefront should handle next, or ~0u when there is none.
+// `r` walks [r0, r1) when the list overflowed.
+__device__ __forceinline__ uint32_t next_dense(const uint32_t* dl, const uint32_t* rc, uint32_t* cursor, uint32_t r0,
+                                               uint32_t r1) {
+    const uint32_t n = dl[0];
+    const uint32_t step = kBlock / kWave;
+    if (n <= kDenseList) {
+        const uint32_t i = *cursor;
+        if (i >= n) return ~0u;
+        *cursor = i + step;
+        return dl[1 + i];
+    }
+    for (uint32_t r = r0 + *cursor; r < r1; r += step) {
+        if (rc[r] == kDense) {
+            *cursor = r - r0 + step;
+            return r;
+        }
+    }
+    return ~0u;
+}
+
+// Copies the bit patterns of a dense region's elements [e0, e1) into this
+// wavefront's kRegion words of LDS, every load issued before the first store, so
+// that the loops over a dense region are not a chain of dependent HBM reads.
+__device__ __forceinline__ void stage_region(const float* rp, uint64_t e0, uint64_t e1, uint32_t* buf) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t v[kRegion / kWave];
+#pragma unroll
+    for (int it = 0; it < kRegion / kWave; it++) {
+        const uint64_t i = e0 + (uint64_t)it * kWave + lane;
+        v[it] = i < e1 ? f2u(rp[i]) : 0u;
+    }
+#pragma unroll
+    for (int it = 0; it < kRegion / kWave; it++) buf[it * kWave + lane] = v[it];
+}
+
+// The regions [r0, r1) of bucket b that block s of kNSub works on.
+__device__ __forceinline__ void block_regions(const Geometry& g, uint32_t b, uint32_t s, uint32_t* r0, uint32_t* r1) {
+    const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
+    const uint32_t per = (nreg + kNSub - 1) / kNSub;
+    *r0 = s * per < nreg ? s * per : nreg;
+    *r1 = *r0 + per < nreg ? *r0 + per : nreg;
+}
+
+// residual <- grad + residual; candidates (key >= lo) are written to their
+// region.  One 8192-element tile per block, tiles in address order, one region
+// per wavefront.  Elements at or above the predicted threshold are stored as
+// 0.0f straight away (their values are in the region's list): a million
+// scattered 4-byte stores after the selection cost more than a tenth of the
+// whole compress, while the streaming store here is free; emit only repairs
+// the few elements between the predicted and the true threshold.  A region
+// that turns out dense puts its values back and stores plain sums from then on.
+// Nothing else happens here: returning atomics and histogram flushes in these
+// 12,000 streaming blocks each cost 7-15 % of the kernel's time when they were
+// tried.
 __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __restrict__ grad, float* residual,
                                                              Geometry g, Workspace w) {
-    __shared__ uint32_t stage[kBlock / kWave][kStage][2];
+    __shared__ uint32_t stage[kBlock / kWave][kRegSlots][2];
     const uint32_t b = blockIdx.y, t = blockIdx.x;
     const uint64_t bn = bucket_count(g, b);
-    const uint64_t e0 = (uint64_t)t * kATile;
-    if (e0 >= bn) return;
-    const float* gp = grad + (uint64_t)b * g.bucket_elems;
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const uint64_t w0 = (uint64_t)t * kATile + (uint64_t)wave * kRegion;  // first element of this wave's region
+    if (w0 >= bn) return;  // whole wavefront; the kernel has no barriers
+    const float* gp = grad + (uint64_t)b * g.bucket_elems + w0;
+    float* rp = residual + (uint64_t)b * g.bucket_elems + w0;
     constexpr int U = 2;
-    constexpr int ROUNDS = kATile / (kBlock * 4 * U);
-    const uint64_t tile_end = (e0 + kATile) < bn ? (e0 + kATile) : bn;
-    const uint64_t nfull = (tile_end - e0) / 4;  // full vectors in this tile
+    constexpr int ROUNDS = kRegion / (kWave * 4 * U);
+    const uint32_t len = (uint32_t)((bn - w0) < (uint64_t)kRegion ? (bn - w0) : (uint64_t)kRegion);
+    const uint32_t nfull = len / 4;  // full vectors in this region
     // The streaming loads of a round are issued one round ahead: round 0's before
     // the bucket parameters are read, round r+1's before round r is processed.
     u4a gv[ROUNDS][U], rv[ROUNDS][U];
     auto issue = [&](int round) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const uint64_t vi = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
+            const uint32_t vi = (uint32_t)(round * U + u) * kWave + lane;
             if (vi < nfull) {
-                gv[round][u] = __builtin_nontemporal_load((const u4u4*)(gp + e0 + vi * 4));
-                rv[round][u] = __builtin_nontemporal_load((const u4u4*)(rp + e0 + vi * 4));
+                gv[round][u] = __builtin_nontemporal_load((const u4u4*)(gp + vi * 4));
+                rv[round][u] = __builtin_nontemporal_load((const u4u4*)(rp + vi * 4));
             }
         }
     };
     issue(0);
     const uint32_t lo_key = w.state[(uint64_t)b * kStateWords + S_LO_KEY];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
-    const uint32_t sub = t % kNSub;
-    uint32_t* sub_cnt = w.sub_count + (uint64_t)b * kNSub + sub;
-    uint32_t* sub_list = w.list + (((uint64_t)b * kNSub + sub) * g.lsub) * 2;
+    const uint32_t that_key = w.state[(uint64_t)b * kStateWords + S_THAT];
+    const uint64_t below = (1ull << lane) - 1ull;
     uint32_t staged = 0;  // wave-uniform
+    bool dense = false;   // wave-uniform: more candidates than slots
 
-    auto flush_stage = [&]() {
-        uint32_t base = 0;
-        if (lane == 0) base = atomicAdd(sub_cnt, staged);
-        base = __shfl(base, 0, kWave);
-        for (uint32_t i = lane; i < staged; i += kWave) {
-            const uint32_t pos = base + i;
-            if (pos < g.lsub) {
-                sub_list[2 * (uint64_t)pos] = stage[wave][i][0];
-                sub_list[2 * (uint64_t)pos + 1] = stage[wave][i][1];
-            }
+    // Appends the lanes' candidates (mask4: which of a lane's four elements) in
+    // index order: lane-major, element-minor.  `cnt` lanes-with-at-least-j
+    // ballots give every lane the number of candidates in the lanes below it.
+    auto append = [&](uint32_t mask4, const u4a& a, uint32_t first_idx) {
+        const uint32_t c = __popc(mask4);
+        uint64_t m = __ballot(c >= 1);
+        if (!m) return;  // wave-uniform
+        uint32_t before = __popcll(m & below), total = __popcll(m);
+#pragma unroll
+        for (uint32_t level = 2; level <= 4; level++) {
+            m = __ballot(c >= level);
+            if (!m) break;  // wave-uniform; nearly always taken at level 2
+            before += __popcll(m & below);
+            total += __popcll(m);
         }
-        staged = 0;
+        if (dense) return;
+        if (staged + total > (uint32_t)kRegSlots) {
+            // the region goes dense: its earlier candidates were stored as zeros where
+            // they reached the predicted threshold; put those values back
+            dense = true;
+            if ((uint32_t)lane < staged && (stage[wave][lane][1] & 0x7FFFFFFFu) >= that_key)
+                residual[(uint64_t)b * g.bucket_elems + stage[wave][lane][0]] = u2f(stage[wave][lane][1]);
+            return;
+        }
+        uint32_t pos = staged + before;
+        while (mask4) {
+            const uint32_t q = (uint32_t)__ffs((int)mask4) - 1u;
+            stage[wave][pos][0] = first_idx + q;
+            stage[wave][pos][1] = q == 0 ? a[0] : (q == 1 ? a[1] : (q == 2 ? a[2] : a[3]));
+            pos++;
+            mask4 &= mask4 - 1u;
+        }
+        staged += total;
     };
 
 #pragma unroll
@@ -579,131 +712,127 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         if (round + 1 < ROUNDS) issue(round + 1);
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const uint64_t vi = (uint64_t)round * (kBlock * U) + (uint64_t)u * kBlock + threadIdx.x;
-            u4a a = {0u, 0u, 0u, 0u};
-            uint32_t mask4 = 0;  // which of this lane's four elements are candidates
+            const uint32_t vi = (uint32_t)(round * U + u) * kWave + lane;
+            u4a a = {0u, 0u, 0u, 0u}, z = {0u, 0u, 0u, 0u};
+            uint32_t mask4 = 0;
             if (vi < nfull) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const float adj = u2f(gv[round][u][q]) + u2f(rv[round][u][q]);
                     a[q] = f2u(adj);
+                    z[q] = key_of(adj) >= that_key ? 0u : a[q];
                     mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
                 }
-                __builtin_nontemporal_store(a, (u4u4*)(rp + e0 + vi * 4));
             }
-            // One staging step per level: every lane that still holds a candidate stages its
-            // lowest one.  About 6 % of the lanes hold one, hardly any holds two, so the
-            // second trip is rare; per-element ballots would run four times on every vector.
-            uint64_t act = __ballot(mask4 != 0);
-            while (act) {  // wave-uniform
-                if (staged + kWave > kStage) flush_stage();
-                if (mask4) {
-                    const uint32_t q = (uint32_t)__ffs((int)mask4) - 1u;
-                    const uint32_t val = q == 0 ? a[0] : (q == 1 ? a[1] : (q == 2 ? a[2] : a[3]));
-                    const uint32_t pos = staged + __popcll(act & ((1ull << lane) - 1ull));
-                    stage[wave][pos][0] = (uint32_t)(e0 + vi * 4) + q;
-                    stage[wave][pos][1] = val;
-                    mask4 &= mask4 - 1u;
-                }
-                staged += (uint32_t)__popcll(act);
-                act = __ballot(mask4 != 0);
-            }
+            append(mask4, a, (uint32_t)w0 + vi * 4);  // may turn the region dense
+            if (vi < nfull) __builtin_nontemporal_store(dense ? a : z, (u4u4*)(rp + vi * 4));
         }
     }
-    // the bucket's last partial vector (bucket length not a multiple of 4)
-    if (tile_end == bn && (bn & 3) && wave == 0) {
-        const uint64_t i = e0 + nfull * 4 + lane;
-        bool c = false;
-        uint32_t bitsv = 0;
-        if (lane < 4 && i < bn) {
-            const float adj = gp[i] + rp[i];
-            rp[i] = adj;
-            bitsv = f2u(adj);
-            c = key_of(adj) >= lo_key;
-        }
-        const uint64_t m = __ballot(c);
-        if (m) {
-            if (staged + kWave > kStage) flush_stage();
-            if (c) {
-                const uint32_t pos = staged + __popcll(m & ((1ull << lane) - 1ull));
-                stage[wave][pos][0] = (uint32_t)i;
-                stage[wave][pos][1] = bitsv;
+    // the bucket's last partial vector (bucket length not a multiple of 4) lies in its last region
+    if (len & 3) {
+        u4a a = {0u, 0u, 0u, 0u};
+        uint32_t mask4 = 0;
+        if (lane == 0) {
+            for (uint32_t q = 0; q < (len & 3); q++) {
+                const float adj = gp[nfull * 4 + q] + rp[nfull * 4 + q];
+                a[q] = f2u(adj);
+                mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
             }
-            staged += (uint32_t)__popcll(m);
+        }
+        append(mask4, a, (uint32_t)w0 + nfull * 4);
+        if (lane == 0) {
+            for (uint32_t q = 0; q < (len & 3); q++)
+                rp[nfull * 4 + q] = (!dense && (a[q] & 0x7FFFFFFFu) >= that_key) ? 0.0f : u2f(a[q]);
         }
     }
-    if (staged) flush_stage();
+    const uint32_t region = (uint32_t)(w0 / kRegion);
+    if (!dense && (uint32_t)lane < staged) {
+        u2a e = {stage[wave][lane][0], stage[wave][lane][1]};
+        *(u2a*)(w.list + (((uint64_t)b * g.regions + region) * kRegSlots + lane) * 2) = e;
+    }
+    if (lane == 0) w.reg_cnt[(uint64_t)b * g.regions + region] = dense ? kDense : staged;
 }
 
-// A block's view of up to 8 * kBlock consecutive (index, bits) entries: all
-// loads are issued before the first use.
-struct EntryChunk {
-    uint32_t idx[8], bits[8];
-    bool valid[8];
-};
-__device__ __forceinline__ EntryChunk load_entries(const uint32_t* l, uint32_t base, uint32_t cnt) {
-    EntryChunk c;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const uint32_t i = base + (uint32_t)j * kBlock + threadIdx.x;
-        c.valid[j] = i < cnt;
-        const uint32_t ii = c.valid[j] ? i : 0u;
-        c.idx[j] = l[2 * (uint64_t)ii];
-        c.bits[j] = l[2 * (uint64_t)ii + 1];
-    }
-    return c;
-}
-
-// Window histogram of a bucket's candidates: one block per sub-list, counts in
+// Window histogram of a bucket's candidates: kNSub blocks per bucket, counts in
 // LDS, one flush per block.
-__global__ __launch_bounds__(kBlock) void k_topk_window_hist(Geometry g, Workspace w) {
+__global__ __launch_bounds__(kBlock) void k_topk_window_hist(const float* residual, Geometry g, Workspace w) {
     __shared__ uint32_t lh[kWinBins];
-    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    __shared__ uint32_t dl[kDenseList + 2];
+    __shared__ uint32_t dreg[kBlock / kWave][kRegion];
+    const uint32_t b = blockIdx.y;
     const uint32_t* st = w.state + (uint64_t)b * kStateWords;
     const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
-    uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
-    if (cnt > g.lsub) cnt = g.lsub;
-    const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
+    uint32_t r0, r1;
+    block_regions(g, b, blockIdx.x, &r0, &r1);
+    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
+    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
     for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
+    if (threadIdx.x == 0) dl[0] = 0;
     __syncthreads();
-    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
-        const EntryChunk c = load_entries(l, base, cnt);
+    for (uint32_t s0 = r0 * kRegSlots; s0 < r1 * kRegSlots; s0 += kChunk * kBlock) {
+        const SlotChunk c = load_slots(rc, lb, s0, r1 * kRegSlots);
+        note_dense(c, dl);
 #pragma unroll
-        for (int j = 0; j < 8; j++)
+        for (int j = 0; j < kChunk; j++)
             if (c.valid[j]) atomicAdd(&lh[window_bin(c.bits[j] & 0x7FFFFFFFu, lo, hi, shift)], 1u);
+    }
+    __syncthreads();
+    if (dl[0]) {  // rare: some region of this block's range is dense
+        const uint64_t bn = bucket_count(g, b);
+        const float* rp = residual + (uint64_t)b * g.bucket_elems;
+        uint32_t cursor = threadIdx.x / kWave;
+        for (uint32_t r; (r = next_dense(dl, rc, &cursor, r0, r1)) != ~0u;) {
+            const uint64_t e0 = (uint64_t)r * kRegion;
+            const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
+            uint32_t* buf = dreg[threadIdx.x / kWave];
+            stage_region(rp, e0, e1, buf);
+            for (uint32_t i = threadIdx.x & (kWave - 1); i < (uint32_t)(e1 - e0); i += kWave) {
+                const uint32_t key = buf[i] & 0x7FFFFFFFu;
+                if (key >= lo) atomicAdd(&lh[window_bin(key, lo, hi, shift)], 1u);
+            }
+        }
     }
     __syncthreads();
     flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kWinBins, kWinBins);
 }
 
-// select, step 1: one block per candidate sub-list.  Finds the window bin that
-// holds the k-th largest key (every block gets the same answer) and copies that
-// bin's candidates to list2 (order irrelevant): the rest of the selection only
-// touches those.
-__global__ __launch_bounds__(kBlock) void k_topk_select1(Geometry g, Workspace w) {
+// select, step 1: finds the window bin that holds the k-th largest key (every
+// block gets the same answer), counts per region the candidates in higher bins
+// (picks for certain) and copies the threshold bin's candidates to list2 (order
+// irrelevant): the rest of the selection only touches those.
+__global__ __launch_bounds__(kBlock) void k_topk_select1(const float* residual, Geometry g, Workspace w) {
     __shared__ uint32_t scratch[kBlock / kWave + 2];
     __shared__ uint32_t gbase;
-    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    __shared__ uint32_t dl[kDenseList + 2];
+    __shared__ uint32_t dreg[kBlock / kWave][kRegion];
+    const uint32_t b = blockIdx.y;
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
+    if (threadIdx.x == 0) dl[0] = 0;  // pick_bin's barriers publish it
     uint32_t need;
     const uint32_t jstar = pick_bin<kWinBins, kBlock>(w.hist_w + (uint64_t)b * kWinBins, bucket_k(g, b), 0, &need, scratch);
-    if (s == 0 && threadIdx.x == 0) { st[S_P0] = jstar; st[S_R0] = need; }
+    if (blockIdx.x == 0 && threadIdx.x == 0) { st[S_P0] = jstar; st[S_R0] = need; }
     // fewer than k candidates, or the threshold lies above the window: fallback
     if (jstar >= (uint32_t)(kWinBins - 1)) return;
-    uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
-    if (cnt > g.lsub) cnt = g.lsub;
-    const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
-    uint32_t* l2 = w.list2 + ((uint64_t)b * kNSub * g.lsub) * 2;
-    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
-        const EntryChunk c = load_entries(l, base, cnt);
+    uint32_t r0, r1;
+    block_regions(g, b, blockIdx.x, &r0, &r1);
+    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
+    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
+    uint32_t* rpick = w.reg_pick + (uint64_t)b * g.regions;
+    uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
+    const int lane = threadIdx.x & (kWave - 1);
+    for (uint32_t s0 = r0 * kRegSlots; s0 < r1 * kRegSlots; s0 += kChunk * kBlock) {
+        const SlotChunk c = load_slots(rc, lb, s0, r1 * kRegSlots);
+        note_dense(c, dl);
         uint32_t mine = 0;
-        bool hit[8];
+        bool hit[kChunk];
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
-            hit[j] = c.valid[j] && window_bin(key, lo, hi, shift) == jstar;
+        for (int j = 0; j < kChunk; j++) {
+            const uint32_t bin = c.valid[j] ? window_bin(c.bits[j] & 0x7FFFFFFFu, lo, hi, shift) : 0u;
+            hit[j] = c.valid[j] && bin == jstar;
             mine += hit[j] ? 1u : 0u;
+            const uint64_t above = __ballot(c.valid[j] && bin > jstar);  // a wavefront = one region
+            if (lane == 0 && c.region[j] < r1) rpick[c.region[j]] = (uint32_t)__popcll(above);
         }
         uint32_t total;
         uint32_t pos = block_exclusive_scan(mine, scratch, &total);
@@ -712,14 +841,50 @@ __global__ __launch_bounds__(kBlock) void k_topk_select1(Geometry g, Workspace w
             __syncthreads();
             pos += gbase;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < kChunk; j++) {
                 if (hit[j]) {
-                    l2[2 * (uint64_t)pos] = c.idx[j];
-                    l2[2 * (uint64_t)pos + 1] = c.bits[j] & 0x7FFFFFFFu;
+                    if (pos < g.lcap2) {
+                        l2[2 * (uint64_t)pos] = c.idx[j];
+                        l2[2 * (uint64_t)pos + 1] = c.bits[j] & 0x7FFFFFFFu;
+                    }
                     pos++;
                 }
             }
             __syncthreads();
+        }
+    }
+    __syncthreads();
+    if (dl[0]) {  // rare
+        const uint64_t bn = bucket_count(g, b);
+        const float* rp = residual + (uint64_t)b * g.bucket_elems;
+        uint32_t cursor = threadIdx.x / kWave;
+        for (uint32_t r; (r = next_dense(dl, rc, &cursor, r0, r1)) != ~0u;) {
+            const uint64_t e0 = (uint64_t)r * kRegion;
+            const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
+            uint32_t above_total = 0;
+            uint32_t* buf = dreg[threadIdx.x / kWave];
+            stage_region(rp, e0, e1, buf);
+            for (uint64_t base = e0; base < e1; base += kWave) {  // wave-uniform trip count
+                const uint64_t i = base + lane;
+                const uint32_t key = i < e1 ? (buf[i - e0] & 0x7FFFFFFFu) : 0u;
+                const uint32_t bin = (i < e1 && key >= lo) ? window_bin(key, lo, hi, shift) : 0u;
+                const bool cand = i < e1 && key >= lo;
+                above_total += (uint32_t)__popcll(__ballot(cand && bin > jstar));
+                const uint64_t hm = __ballot(cand && bin == jstar);
+                if (hm) {
+                    uint32_t base2 = 0;
+                    if (lane == 0) base2 = atomicAdd(st + S_N2, (uint32_t)__popcll(hm));
+                    base2 = __shfl(base2, 0, kWave);
+                    if (cand && bin == jstar) {
+                        const uint32_t pos = base2 + (uint32_t)__popcll(hm & ((1ull << lane) - 1ull));
+                        if (pos < g.lcap2) {
+                            l2[2 * (uint64_t)pos] = (uint32_t)i;
+                            l2[2 * (uint64_t)pos + 1] = key;
+                        }
+                    }
+                }
+            }
+            if (lane == 0) rpick[r] = above_total;
         }
     }
 }
@@ -775,9 +940,30 @@ __device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uin
     }
 }
 
-// select, step 2: one block per bucket.  Validates the candidate lists, finishes
-// the radix select on list2 (keys of one window bin: 24 bits at most remain)
-// and resolves ties by index.
+// Puts back the values pass A replaced by 0.0f (listed candidates with key >=
+// the predicted threshold) so that the exact fallback sees the plain sums.
+// Called by all threads of a select2 block.
+__device__ void restore_prezeroed(float* residual, const Geometry& g, const Workspace& w, uint32_t b) {
+    const uint32_t that_key = w.state[(uint64_t)b * kStateWords + S_THAT];
+    const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
+    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
+    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    for (uint32_t slot = threadIdx.x; slot < nreg * kRegSlots; slot += kSelThreads) {
+        const uint32_t cnt = rc[slot / kRegSlots];
+        if (cnt == kDense || (slot % kRegSlots) >= cnt) continue;
+        const uint32_t idx = lb[2 * (uint64_t)slot], bitsv = lb[2 * (uint64_t)slot + 1];
+        if ((bitsv & 0x7FFFFFFFu) >= that_key) rp[idx] = u2f(bitsv);
+    }
+    __threadfence();
+    __syncthreads();
+}
+
+// select, step 2: one block per bucket.  Checks that the threshold lies inside
+// the window and list2 is complete (else the bucket takes the exact fallback),
+// finishes the radix select on list2 (keys of one window bin: 24 bits at most
+// remain), resolves ties by index, adds the threshold bin's picks to the
+// per-region pick counts and turns those into each region's offset in the payload.
 __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, Geometry g, Workspace w,
                                                               uint8_t* wire, uint64_t wire_stride) {
     __shared__ uint32_t lh[kBins0];
@@ -786,21 +972,18 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     const uint32_t jstar = st[S_P0];
     uint32_t want = st[S_R0];
-    uint32_t over = 0;
-    if (threadIdx.x < kNSub) over = w.sub_count[(uint64_t)b * kNSub + threadIdx.x] > g.lsub ? 1u : 0u;
-    uint32_t any_over;
-    block_exclusive_scan_n<kSelThreads>(over, scratch, &any_over);
-    if (any_over || jstar >= (uint32_t)(kWinBins - 1)) {
-        // incomplete candidate lists or threshold outside the window (rare): this block
-        // runs the whole exact selection of the bucket; S_OK stays 0, so mark and emit skip it
+    const uint32_t count2 = st[S_N2];
+    if (jstar >= (uint32_t)(kWinBins - 1) || count2 > g.lcap2) {
+        // threshold outside the window, or more keys in its bin than list2 holds (rare):
+        // this block runs the whole exact selection of the bucket; S_OK stays 0, so emit skips it
+        restore_prezeroed(residual, g, w, b);
         bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
         return;
     }
 
-    const uint32_t* l2 = w.list2 + ((uint64_t)b * kNSub * g.lsub) * 2;
-    const uint32_t count2 = st[S_N2];
+    const uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
     const uint32_t bin_lo = st[S_LO_KEY] + (jstar << st[S_SHIFT]);  // smallest key of the bin
-    uint32_t vprefix = 0;  // key - bin_lo: up to 24 bits, selected as 4 + 10 + 10
+    uint32_t vprefix = 0;  // key - bin_lo: up to 30 bits, selected as 10 + 10 + 10
     for (int r = 0; r < 3; r++) {
         const int shift = 20 - 10 * r;
         const int hs = shift + 10;
@@ -848,114 +1031,116 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
         }
         istar = iprefix;
     }
+
+    // picks inside the threshold bin join their regions' counts; then an exclusive
+    // scan over the regions gives each region's first position in the payload
+    uint32_t* rpick = w.reg_pick + (uint64_t)b * g.regions;
+    for (uint32_t i = threadIdx.x; i < count2; i += kSelThreads) {
+        const uint32_t idx = l2[2 * (uint64_t)i], key = l2[2 * (uint64_t)i + 1];
+        if (key > T || (key == T && idx <= istar)) atomicAdd(&rpick[idx / kRegion], 1u);
+    }
+    __threadfence();
+    __syncthreads();
+    const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
+    const uint32_t per = (nreg + kSelThreads - 1) / kSelThreads;
+    const uint32_t first = threadIdx.x * per;
+    uint32_t sum = 0;
+    for (uint32_t j = 0; j < per; j++)
+        if (first + j < nreg) sum += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t total;
+    uint32_t run = block_exclusive_scan_n<kSelThreads>(sum, scratch, &total);
+    uint32_t* roff = w.reg_off + (uint64_t)b * g.regions;
+    for (uint32_t j = 0; j < per; j++) {
+        if (first + j < nreg) {
+            roff[first + j] = run;
+            run += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     if (threadIdx.x == 0) {
         st[S_T] = T;
         st[S_NEED] = need2;
         st[S_ISTAR] = istar;
-        st[S_OK] = 1;
+        st[S_OK] = total == bucket_k(g, b) ? 1u : 0u;
+    }
+    if (total != bucket_k(g, b)) {  // uniform; cannot happen with consistent lists
+        __syncthreads();
+        restore_prezeroed(residual, g, w, b);
+        bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
     }
 }
 
-// One block per candidate sub-list.  A sub-list holds the candidates of the
-// pass-A tiles t = s, s + kNSub, ..., so this block sees every pick of those
-// 8192-element tiles.  It builds the tiles' pick bitmaps in LDS, derives every
-// pick's rank inside its tile from them (popcount prefix), writes the picks of
-// each tile, in index order, as one contiguous run of the bucket's staging
-// list, zeroes the residual at the picks, and records (offset, count) per tile.
-// The emit kernel then only concatenates the runs.
-__global__ __launch_bounds__(kBlock) void k_topk_mark(float* residual, Geometry g, Workspace w) {
-    // dynamic LDS, sized by the launch for ceil(etiles / kNSub) tiles (at most kMarkTiles):
-    // bitmap words, per-word pick prefix, per-tile count and offset
-    extern __shared__ uint32_t mark_lds[];
-    const uint32_t tmax = (g.etiles + kNSub - 1) / kNSub;
-    uint32_t* bm = mark_lds;
-    uint32_t* pre = bm + tmax * (kETile / 32);  // picks of the tile before this word
-    uint32_t* tcount = pre + tmax * (kETile / 32);
-    uint32_t* toff = tcount + tmax;
-    const uint32_t b = blockIdx.y, s = blockIdx.x;
-    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    if (!st[S_OK]) return;
-    const uint32_t T = st[S_T], istar = st[S_ISTAR];
-    const uint32_t ntiles = s < g.etiles ? (g.etiles - s + kNSub - 1) / kNSub : 0u;  // tiles of this sub-list
-    for (uint32_t i = threadIdx.x; i < ntiles * (kETile / 32); i += kBlock) bm[i] = 0;
-    __syncthreads();
-    uint32_t cnt = w.sub_count[(uint64_t)b * kNSub + s];
-    if (cnt > g.lsub) cnt = g.lsub;
-    const uint32_t* l = w.list + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
-    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
-        const EntryChunk c = load_entries(l, base, cnt);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
-            if (c.valid[j] && (key > T || (key == T && c.idx[j] <= istar))) {
-                const uint32_t word = (c.idx[j] / kETile / kNSub) * (kETile / 32) + ((c.idx[j] % kETile) >> 5);
-                atomicOr(&bm[word], 1u << (c.idx[j] & 31));
-            }
-        }
-    }
-    __syncthreads();
-    const int lane = threadIdx.x & (kWave - 1);
-    for (uint32_t j = threadIdx.x / kWave; j < ntiles; j += kBlock / kWave) {  // one wavefront per tile
-        const u4a v = ((const u4a*)(bm + j * (kETile / 32)))[lane];
-        const uint32_t c0 = __popc(v[0]), c1 = __popc(v[1]), c2 = __popc(v[2]), c3 = __popc(v[3]);
-        const uint32_t inc = wave_inclusive_scan(c0 + c1 + c2 + c3);
-        const uint32_t ex = inc - (c0 + c1 + c2 + c3);
-        u4a p = {ex, ex + c0, ex + c0 + c1, ex + c0 + c1 + c2};
-        ((u4a*)(pre + j * (kETile / 32)))[lane] = p;
-        if (lane == kWave - 1) tcount[j] = inc;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t run = 0;
-        for (uint32_t j = 0; j < ntiles; j++) { toff[j] = run; run += tcount[j]; }
-    }
-    __syncthreads();
-    if (threadIdx.x < ntiles) {
-        const uint32_t tile = s + threadIdx.x * kNSub;
-        w.etile_count[(uint64_t)b * g.etiles + tile] = tcount[threadIdx.x];
-        w.etile_off[(uint64_t)b * g.etiles + tile] = toff[threadIdx.x];
-    }
-    uint32_t* stg = w.list2 + (((uint64_t)b * kNSub + s) * g.lsub) * 2;
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
-    for (uint32_t base = 0; base < cnt; base += 8 * kBlock) {
-        const EntryChunk c = load_entries(l, base, cnt);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
-            if (c.valid[j] && (key > T || (key == T && c.idx[j] <= istar))) {
-                const uint32_t tj = c.idx[j] / kETile / kNSub;
-                const uint32_t word = tj * (kETile / 32) + ((c.idx[j] % kETile) >> 5);
-                const uint32_t rank = pre[word] + __popc(bm[word] & ((1u << (c.idx[j] & 31)) - 1u));
-                const uint32_t pos = toff[tj] + rank;
-                stg[2 * (uint64_t)pos] = c.idx[j];
-                stg[2 * (uint64_t)pos + 1] = c.bits[j];
-                rp[c.idx[j]] = 0.0f;
-            }
-        }
-    }
-}
-
-// Concatenates the tiles' runs in tile order: one wavefront per tile.
-__global__ __launch_bounds__(kBlock) void k_topk_emit_fast(Geometry g, Workspace w, uint8_t* wire,
+// Writes the payload: the picks of a region are its candidates with key > T, or
+// key == T and index <= istar, already in index order; they go to the region's
+// offset in pick order.  The residual already holds 0.0f where pass A predicted
+// a pick; picks it missed are zeroed and wrongly predicted ones get their value
+// back.  A wavefront handles one region at a time.
+__global__ __launch_bounds__(kBlock) void k_topk_emit_fast(float* residual, Geometry g, Workspace w, uint8_t* wire,
                                                            uint64_t wire_stride) {
     const uint32_t b = blockIdx.y;
-    if (!w.state[(uint64_t)b * kStateWords + S_OK]) return;
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t t = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    if (!st[S_OK]) return;
+    const uint32_t T = st[S_T], istar = st[S_ISTAR], that_key = st[S_THAT];
+    uint32_t r0, r1;
+    block_regions(g, b, blockIdx.x, &r0, &r1);
+    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
+    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
+    const uint32_t* roff = w.reg_off + (uint64_t)b * g.regions;
     uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
-    if (t == 0 && lane == 0) out[0] = bucket_k(g, b);
-    if (t >= g.etiles) return;
-    const uint32_t* ec = w.etile_count + (uint64_t)b * g.etiles;
-    const uint32_t cnt = ec[t];
-    const uint32_t off = w.etile_off[(uint64_t)b * g.etiles + t];
-    uint32_t base = 0;
-    for (uint32_t i = lane; i < t; i += kWave) base += ec[i];
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
+    const int lane = threadIdx.x & (kWave - 1);
+    __shared__ uint32_t dl[kDenseList + 2];
+    __shared__ uint32_t dreg[kBlock / kWave][kRegion];
+    if (threadIdx.x == 0) dl[0] = 0;
+    __syncthreads();
+    for (uint32_t s0 = r0 * kRegSlots; s0 < r1 * kRegSlots; s0 += kChunk * kBlock) {
+        uint32_t off[kChunk];
 #pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) base += __shfl_xor(base, d, kWave);
-    const uint32_t* src = w.list2 + ((((uint64_t)b * kNSub + (t % kNSub)) * g.lsub) + off) * 2;
-    for (uint32_t i = lane; i < cnt; i += kWave) {
-        out[1 + 2 * (uint64_t)(base + i)] = src[2 * (uint64_t)i];
-        out[2 + 2 * (uint64_t)(base + i)] = src[2 * (uint64_t)i + 1];
+        for (int j = 0; j < kChunk; j++) {
+            const uint32_t r = (s0 + (uint32_t)j * kBlock + threadIdx.x) / kRegSlots;
+            off[j] = r < r1 ? roff[r] : 0u;
+        }
+        const SlotChunk c = load_slots(rc, lb, s0, r1 * kRegSlots);
+        note_dense(c, dl);
+#pragma unroll
+        for (int j = 0; j < kChunk; j++) {
+            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
+            const bool pick = c.valid[j] && (key > T || (key == T && c.idx[j] <= istar));
+            const uint64_t m = __ballot(pick);
+            if (pick) {
+                const uint32_t pos = off[j] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+                u2a e = {c.idx[j], c.bits[j]};
+                *(u2a4*)(out + 1 + 2 * (uint64_t)pos) = e;
+            }
+            // pass A stored 0.0f for key >= predicted threshold; repair where the prediction was wrong
+            if (c.valid[j] && pick != (key >= that_key)) rp[c.idx[j]] = pick ? 0.0f : u2f(c.bits[j]);
+        }
+    }
+    __syncthreads();
+    if (dl[0]) {  // rare
+        const uint64_t bn = bucket_count(g, b);
+        uint32_t cursor = threadIdx.x / kWave;
+        for (uint32_t r; (r = next_dense(dl, rc, &cursor, r0, r1)) != ~0u;) {
+            const uint64_t e0 = (uint64_t)r * kRegion;
+            const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
+            uint32_t pos0 = roff[r];
+            uint32_t* buf = dreg[threadIdx.x / kWave];
+            stage_region(rp, e0, e1, buf);
+            for (uint64_t base = e0; base < e1; base += kWave) {  // wave-uniform trip count
+                const uint64_t i = base + lane;
+                const uint32_t bitsv = i < e1 ? buf[i - e0] : 0u;
+                const uint32_t key = bitsv & 0x7FFFFFFFu;
+                const bool pick = i < e1 && (key > T || (key == T && (uint32_t)i <= istar));
+                const uint64_t m = __ballot(pick);
+                if (pick) {
+                    const uint32_t pos = pos0 + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+                    out[1 + 2 * (uint64_t)pos] = (uint32_t)i;
+                    out[2 + 2 * (uint64_t)pos] = bitsv;
+                    rp[i] = 0.0f;
+                }
+                pos0 += (uint32_t)__popcll(m);
+            }
+        }
     }
 }
 
@@ -965,13 +1150,13 @@ uint64_t align4(uint64_t words) { return (words + 3) & ~uint64_t(3); }
 
 uint64_t zeroed_words(const Geometry& g) {
     return align4((uint64_t)g.nbuckets * kHistWords) + align4((uint64_t)g.nbuckets * kWinBins) +
-           align4((uint64_t)g.nbuckets * kStateWords) + align4((uint64_t)g.nbuckets * kNSub);
+           align4((uint64_t)g.nbuckets * kStateWords);
 }
 
 uint64_t workspace_words(const Geometry& g) {
-    return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.etiles) +
-           2 * align4((uint64_t)g.nbuckets * g.tiles) +
-           2 * align4((uint64_t)g.nbuckets * kNSub * g.lsub * 2);
+    return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) +
+           3 * align4((uint64_t)g.nbuckets * g.regions) +
+           align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2) + align4((uint64_t)g.nbuckets * g.lcap2 * 2);
 }
 
 Workspace carve(void* base, const Geometry& g) {
@@ -980,12 +1165,12 @@ Workspace carve(void* base, const Geometry& g) {
     w.hist = p;        p += align4((uint64_t)g.nbuckets * kHistWords);
     w.hist_w = p;      p += align4((uint64_t)g.nbuckets * kWinBins);
     w.state = p;       p += align4((uint64_t)g.nbuckets * kStateWords);
-    w.sub_count = p;   p += align4((uint64_t)g.nbuckets * kNSub);
-    w.etile_count = p; p += align4((uint64_t)g.nbuckets * g.etiles);
-    w.etile_off = p;   p += align4((uint64_t)g.nbuckets * g.etiles);
     w.tile_gt = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
     w.tile_eq = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
-    w.list = p;        p += align4((uint64_t)g.nbuckets * kNSub * g.lsub * 2);
+    w.reg_cnt = p;     p += align4((uint64_t)g.nbuckets * g.regions);
+    w.reg_pick = p;    p += align4((uint64_t)g.nbuckets * g.regions);
+    w.reg_off = p;     p += align4((uint64_t)g.nbuckets * g.regions);
+    w.list = p;        p += align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2);
     w.list2 = p;
     return w;
 }
@@ -1002,11 +1187,12 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     g->tiles = (uint32_t)((bucket_elems + kTile - 1) / kTile);
     g->k_full = mccl_hip_topk_k(bucket_elems, ratio);
     g->k_last = mccl_hip_topk_k(n_total - (nb - 1) * bucket_elems, ratio);
-    g->etiles = (uint32_t)((bucket_elems + kETile - 1) / kETile);
-    // candidate capacity: 4 k + 4096 + n/256 entries per bucket, never more than the bucket
-    uint64_t cap = 4 * (uint64_t)g->k_full + 4096 + bucket_elems / 256;
-    if (cap > bucket_elems + kNSub) cap = bucket_elems + kNSub;
-    g->lsub = (uint32_t)((cap + kNSub - 1) / kNSub);
+    g->regions = (uint32_t)((bucket_elems + kATile - 1) / kATile) * (kATile / kRegion);
+    // list2 holds the candidates of one window bin (1/256 of about 1.7 k in the expected
+    // case); 2 k + 4096 entries leave room for heavy ties, never more than the bucket
+    uint64_t cap = 2 * (uint64_t)g->k_full + 4096;
+    if (cap > bucket_elems) cap = bucket_elems;
+    g->lcap2 = (uint32_t)cap;
     return true;
 }
 
@@ -1054,8 +1240,7 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     void* aligned = (void*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
     Workspace w = carve(aligned, g);
     const int path = tuning().topk_path;  // 0 auto, 1 exact path only, 2 fast path at any size
-    const bool fits = (uint64_t)g.etiles <= (uint64_t)kMarkTiles * kNSub;  // mark keeps a sub-list's bitmap in LDS
-    const bool fast = fits && (path == 2 || (path == 0 && g.bucket_elems >= kFastMinBucket));
+    const bool fast = path == 2 || (path == 0 && g.bucket_elems >= kFastMinBucket);
 
     const uint64_t cap = (uint64_t)device_info().num_cus * (uint64_t)tuning().fold_blocks_per_cu;
     const uint64_t nvec = g.bucket_elems / 4;
@@ -1067,13 +1252,10 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
         k_topk_sample<<<g.nbuckets, kSelThreads, 0, st>>>(grad, residual, g, w);
         const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
-        k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
-        k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(g, w);
+        k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
+        k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
         k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
-        const uint32_t tmax = (g.etiles + kNSub - 1) / kNSub;
-        const size_t mark_lds = (size_t)tmax * (2 * (kETile / 32) + 2) * sizeof(uint32_t);
-        k_topk_mark<<<dim3(kNSub, g.nbuckets), kBlock, mark_lds, st>>>(residual, g, w);
-        k_topk_emit_fast<<<dim3((g.etiles + 3) / 4, g.nbuckets), kBlock, 0, st>>>(g, w, (uint8_t*)wire, wire_stride);
+        k_topk_emit_fast<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
     } else {
         const uint64_t zw = zeroed_words(g);
         k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);
