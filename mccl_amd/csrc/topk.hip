@@ -984,7 +984,9 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     const uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
     const uint32_t bin_lo = st[S_LO_KEY] + (jstar << st[S_SHIFT]);  // smallest key of the bin
     uint32_t vprefix = 0;  // key - bin_lo: up to 30 bits, selected as 10 + 10 + 10
-    for (int r = 0; r < 3; r++) {
+    // a window bin spans 2^S_SHIFT keys: rounds whose digits lie wholly above that are skipped
+    const int first_round = st[S_SHIFT] <= 10 ? 2 : (st[S_SHIFT] <= 20 ? 1 : 0);
+    for (int r = first_round; r < 3; r++) {
         const int shift = 20 - 10 * r;
         const int hs = shift + 10;
         for (int i = threadIdx.x; i < kBinsR; i += kSelThreads) lh[i] = 0;
@@ -1044,16 +1046,34 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
     const uint32_t per = (nreg + kSelThreads - 1) / kSelThreads;
     const uint32_t first = threadIdx.x * per;
-    uint32_t sum = 0;
-    for (uint32_t j = 0; j < per; j++)
-        if (first + j < nreg) sum += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t total;
-    uint32_t run = block_exclusive_scan_n<kSelThreads>(sum, scratch, &total);
     uint32_t* roff = w.reg_off + (uint64_t)b * g.regions;
-    for (uint32_t j = 0; j < per; j++) {
-        if (first + j < nreg) {
-            roff[first + j] = run;
-            run += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t total;
+    constexpr uint32_t kHeld = 8;  // counts a thread keeps in registers between the two sweeps
+    if (per <= kHeld) {
+        uint32_t held[kHeld];
+#pragma unroll
+        for (uint32_t j = 0; j < kHeld; j++)
+            held[j] = (j < per && first + j < nreg)
+                          ? __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+        uint32_t sum = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < kHeld; j++) sum += held[j];
+        uint32_t run = block_exclusive_scan_n<kSelThreads>(sum, scratch, &total);
+#pragma unroll
+        for (uint32_t j = 0; j < kHeld; j++) {
+            if (j < per && first + j < nreg) roff[first + j] = run;
+            run += held[j];
+        }
+    } else {
+        uint32_t sum = 0;
+        for (uint32_t j = 0; j < per; j++)
+            if (first + j < nreg) sum += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t run = block_exclusive_scan_n<kSelThreads>(sum, scratch, &total);
+        for (uint32_t j = 0; j < per; j++) {
+            if (first + j < nreg) {
+                roff[first + j] = run;
+                run += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
     if (threadIdx.x == 0) {
