@@ -173,6 +173,54 @@ __device__ __forceinline__ uint32_t pick_bin(const uint32_t* h, uint32_t remaini
     return bin;
 }
 
+// pick_bin for NR histograms (or NR ranks in one histogram) at once, in the same
+// three barriers.  remaining[z] == 0 switches rank z off (bin[z] = BINS).
+// scratch: NR * (THREADS / kWave + 2) words.
+template <int BINS, int THREADS, int NR>
+__device__ __forceinline__ void pick_bins(const uint32_t* const (&h)[NR], const uint32_t (&remaining)[NR],
+                                          uint32_t (&bin)[NR], uint32_t (&left)[NR], uint32_t* scratch) {
+    constexpr int PER = (BINS + THREADS - 1) / THREADS;
+    constexpr int NW = THREADS / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    uint32_t c[NR][PER], sum[NR], inc[NR];
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        sum[z] = 0;
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int r = threadIdx.x * PER + j;  // reversed bin number
+            c[z][j] = r < BINS ? h[z][BINS - 1 - r] : 0u;
+            sum[z] += c[z][j];
+        }
+        inc[z] = wave_inclusive_scan(sum[z]);
+        if (lane == kWave - 1) scratch[z * NW + wave] = inc[z];
+    }
+    uint32_t* res = scratch + NR * NW;
+    if (threadIdx.x < NR) { res[2 * threadIdx.x] = BINS; res[2 * threadIdx.x + 1] = 0; }
+    __syncthreads();
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        uint32_t above = inc[z] - sum[z];
+        for (int w2 = 0; w2 < wave; w2++) above += scratch[z * NW + w2];
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            if (above < remaining[z] && remaining[z] <= above + c[z][j]) {
+                res[2 * z] = BINS - 1 - (threadIdx.x * PER + j);
+                res[2 * z + 1] = remaining[z] - above;
+            }
+            above += c[z][j];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        bin[z] = res[2 * z];
+        left[z] = res[2 * z + 1];
+    }
+    __syncthreads();
+}
+
 // ================================ exact path ======================================
 
 // residual <- grad + residual, histogram of key[30:20].
@@ -432,16 +480,17 @@ __device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32
 }
 
 // One block per bucket.  Loads kSample evenly spread elements of grad + residual
-// into LDS and radix-selects (11 + 10 + 10 key bits, both ranks in the same
-// sweeps) the keys of sample ranks
-//     r_hi = ks - 6 sqrt(ks) - 16   and   r_lo = ks + 6 sqrt(ks) + 16,
-// ks = k * S / n being the expected number of sampled elements among the top k.
+// into LDS and radix-selects (11 + 10 key bits, all ranks in the same sweeps)
+// the keys of sample ranks
+//     r_hi = ks - 6 sqrt(ks) - 16,   r_lo = ks + 6 sqrt(ks) + 16   and   ks,
+// ks = k * S / n being the expected number of sampled elements among the top k:
+// the two ends of the candidate window and the predicted threshold.
 __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __restrict__ grad,
                                                              const float* __restrict__ residual, Geometry g,
                                                              Workspace w) {
     __shared__ uint32_t keys[kSample];
     __shared__ uint32_t lh[3][kBinsR];
-    __shared__ uint32_t scratch[kSelThreads / kWave + 2];
+    __shared__ uint32_t scratch[3 * (kSelThreads / kWave + 2)];
     const uint32_t b = blockIdx.x;
     // this bucket's accumulators for the kernels that follow start at zero
     for (int i = threadIdx.x; i < kWinBins; i += kSelThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
@@ -480,36 +529,45 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     rank[2] = ks >= 1.0f ? (uint32_t)ks : 1u;
     uint32_t prefix[NR] = {0u, 0u, 0u}, want[NR] = {rank[0], rank[1], rank[2]};
     const bool active[NR] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S, rank[2] <= S};
-    const int shifts[3] = {20, 10, 0};
+    // Two rounds, 11 + 10 key bits: the selected keys are exact to 2^-13 of their value,
+    // far finer than the sampling noise the window margins allow for.  The ten low bits
+    // are filled so that the window only widens.
     __syncthreads();
-    for (int r = 0; r < 3; r++) {
+    for (int r = 0; r < 2; r++) {
         // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves all ranks
         uint32_t* h0 = &lh[0][0];
         for (int i = threadIdx.x; i < NR * kBinsR; i += kSelThreads) h0[i] = 0;
         __syncthreads();
-        const int shift = shifts[r];
         for (uint32_t i = threadIdx.x; i < S; i += kSelThreads) {
             const uint32_t key = keys[i];
             if (r == 0) {
                 atomicAdd(&h0[key >> 20], 1u);
             } else {
-                const int hs = shift + 10;
 #pragma unroll
                 for (int z = 0; z < NR; z++)
-                    if (active[z] && (key >> hs) == (prefix[z] >> hs)) atomicAdd(&lh[z][(key >> shift) & (kBinsR - 1)], 1u);
+                    if (active[z] && (key >> 20) == (prefix[z] >> 20)) atomicAdd(&lh[z][(key >> 10) & (kBinsR - 1)], 1u);
             }
         }
         __syncthreads();
+        uint32_t rem[NR], bin[NR], left[NR];
+#pragma unroll
+        for (int z = 0; z < NR; z++) rem[z] = active[z] ? want[z] : 0u;
+        if (r == 0) {
+            const uint32_t* const hs[NR] = {h0, h0, h0};
+            pick_bins<kBins0, kSelThreads, NR>(hs, rem, bin, left, scratch);
+        } else {
+            const uint32_t* const hs[NR] = {lh[0], lh[1], lh[2]};
+            pick_bins<kBinsR, kSelThreads, NR>(hs, rem, bin, left, scratch);
+        }
 #pragma unroll
         for (int z = 0; z < NR; z++) {
             if (!active[z]) continue;
-            uint32_t left, bin;
-            if (r == 0) bin = pick_bin<kBins0, kSelThreads>(h0, want[z], 0, &left, scratch);
-            else bin = pick_bin<kBinsR, kSelThreads>(lh[z], want[z], 0, &left, scratch);
-            prefix[z] |= bin << shift;
-            want[z] = left;
+            prefix[z] |= bin[z] << (r == 0 ? 20 : 10);
+            want[z] = left[z];
         }
     }
+    prefix[0] |= 0x3FFu;  // upper end of the window: rounded up
+    prefix[2] |= 0x200u;  // predicted threshold: middle of its 1024-key cell
     if (threadIdx.x == 0) {
         const uint32_t lo = active[1] ? prefix[1] : 0u;
         uint32_t hi = active[0] ? prefix[0] : 0x7FFFFFFFu;
