@@ -63,6 +63,7 @@ static_assert(kRegSlots == kWave, "a wavefront reads a region's slots in one go"
 constexpr uint32_t kDense = 0xFFFFFFFFu;  // region count: more candidates than slots, read the residual range itself
 constexpr int kNSub = 64;      // fast path: blocks per bucket in the kernels that walk the regions
 constexpr int kSelThreads = 1024;
+constexpr int kSampleThreads = 1024;  // sample kernel (256 threads measured slower: 21 vs 15.5 us)
 constexpr uint64_t kFastMinBucket = 1u << 18;
 constexpr int kSample = 12288;  // fast path: sampled elements per bucket (12 per select thread)
 
@@ -485,15 +486,15 @@ __device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32
 //     r_hi = ks - 6 sqrt(ks) - 16,   r_lo = ks + 6 sqrt(ks) + 16   and   ks,
 // ks = k * S / n being the expected number of sampled elements among the top k:
 // the two ends of the candidate window and the predicted threshold.
-__global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __restrict__ grad,
+__global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __restrict__ grad,
                                                              const float* __restrict__ residual, Geometry g,
                                                              Workspace w) {
     __shared__ uint32_t keys[kSample];
     __shared__ uint32_t lh[3][kBinsR];
-    __shared__ uint32_t scratch[3 * (kSelThreads / kWave + 2)];
+    __shared__ uint32_t scratch[3 * (kSampleThreads / kWave + 2)];
     const uint32_t b = blockIdx.x;
     // this bucket's accumulators for the kernels that follow start at zero
-    for (int i = threadIdx.x; i < kWinBins; i += kSelThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
+    for (int i = threadIdx.x; i < kWinBins; i += kSampleThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
     if (threadIdx.x < kStateWords) w.state[(uint64_t)b * kStateWords + threadIdx.x] = 0;
     const uint64_t bn = bucket_count(g, b);
     const float* gp = grad + (uint64_t)b * g.bucket_elems;
@@ -503,18 +504,18 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     // sampled in runs of 8 vectors (one 128-byte line per array), runs evenly spread
     const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)(nvec & ~7ull) : (uint32_t)SV;
     const uint64_t stride = nsv ? (nvec / (nsv / 8)) : 8;  // vectors between run starts (>= 8)
-    u4a gv[SV / kSelThreads], rv[SV / kSelThreads];
+    u4a gv[SV / kSampleThreads], rv[SV / kSampleThreads];
 #pragma unroll
-    for (int j = 0; j < SV / kSelThreads; j++) {
-        const uint32_t i = (uint32_t)j * kSelThreads + threadIdx.x;
+    for (int j = 0; j < SV / kSampleThreads; j++) {
+        const uint32_t i = (uint32_t)j * kSampleThreads + threadIdx.x;
         const uint32_t ii = i < nsv ? i : 0;
         const uint64_t v = (uint64_t)(ii >> 3) * stride + (ii & 7);
         gv[j] = nsv ? *(const u4u4*)(gp + v * 4) : u4a{0u, 0u, 0u, 0u};
         rv[j] = nsv ? *(const u4u4*)(rp + v * 4) : u4a{0u, 0u, 0u, 0u};
     }
 #pragma unroll
-    for (int j = 0; j < SV / kSelThreads; j++) {
-        const uint32_t i = (uint32_t)j * kSelThreads + threadIdx.x;
+    for (int j = 0; j < SV / kSampleThreads; j++) {
+        const uint32_t i = (uint32_t)j * kSampleThreads + threadIdx.x;
 #pragma unroll
         for (int q = 0; q < 4; q++) keys[4 * i + q] = i < nsv ? key_of(u2f(gv[j][q]) + u2f(rv[j][q])) : 0u;
     }
@@ -536,9 +537,9 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
     for (int r = 0; r < 2; r++) {
         // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves all ranks
         uint32_t* h0 = &lh[0][0];
-        for (int i = threadIdx.x; i < NR * kBinsR; i += kSelThreads) h0[i] = 0;
+        for (int i = threadIdx.x; i < NR * kBinsR; i += kSampleThreads) h0[i] = 0;
         __syncthreads();
-        for (uint32_t i = threadIdx.x; i < S; i += kSelThreads) {
+        for (uint32_t i = threadIdx.x; i < S; i += kSampleThreads) {
             const uint32_t key = keys[i];
             if (r == 0) {
                 atomicAdd(&h0[key >> 20], 1u);
@@ -554,10 +555,10 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_sample(const float* __rest
         for (int z = 0; z < NR; z++) rem[z] = active[z] ? want[z] : 0u;
         if (r == 0) {
             const uint32_t* const hs[NR] = {h0, h0, h0};
-            pick_bins<kBins0, kSelThreads, NR>(hs, rem, bin, left, scratch);
+            pick_bins<kBins0, kSampleThreads, NR>(hs, rem, bin, left, scratch);
         } else {
             const uint32_t* const hs[NR] = {lh[0], lh[1], lh[2]};
-            pick_bins<kBinsR, kSelThreads, NR>(hs, rem, bin, left, scratch);
+            pick_bins<kBinsR, kSampleThreads, NR>(hs, rem, bin, left, scratch);
         }
 #pragma unroll
         for (int z = 0; z < NR; z++) {
@@ -1327,7 +1328,7 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     const uint32_t bx_r = clamp_u32(bx < need_r ? bx : need_r, 1, 65535);
     const uint32_t bx_t = clamp_u32(bx < g.tiles ? bx : g.tiles, 1, 65535);
     if (fast) {
-        k_topk_sample<<<g.nbuckets, kSelThreads, 0, st>>>(grad, residual, g, w);
+        k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(grad, residual, g, w);
         const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
         k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
