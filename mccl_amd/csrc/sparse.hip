@@ -21,6 +21,7 @@ namespace mcclhip {
 
 namespace {
 
+constexpr int kAccThreads = 512;  // threads per block of the accumulate kernel with bounds
 constexpr int kAccTile = 8192;  // output elements per block, accumulated in LDS (32 KiB)
 
 __global__ __launch_bounds__(kBlock) void k_fill_zero(float* p, uint64_t n) {
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(kBlock) void k_sparse_bounds(WirePtrs wires, int ws
 // Accumulate with precomputed bounds: every block reads its 2 * ws bounds with one
 // load per lane, then issues the loads of all its pairs (every rank) before the
 // first LDS add; the adds run rank by rank.
-__global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint64_t n_total,
+__global__ __launch_bounds__(kAccThreads) void k_sparse_accumulate_b(float* acc, uint64_t n_total,
                                                                 uint64_t bucket_elems, WirePtrs wires, int ws,
                                                                 uint64_t wire_stride, uint32_t tiles,
                                                                 const uint32_t* start, int apply_scale,
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint
         if (v > kmax) v = kmax;  // stale bound of a malformed payload: stay inside the buffer
         if (threadIdx.x < ws) lo_s[r] = v; else hi_s[r] = v;
     }
-    for (int i = threadIdx.x; i < kAccTile; i += kBlock) tile[i] = 0.0f;
+    for (int i = threadIdx.x; i < kAccTile; i += kAccThreads) tile[i] = 0.0f;
     __syncthreads();
     constexpr int RB = 8;  // ranks whose pairs are in flight together
     for (int r0 = 0; r0 < ws; r0 += RB) {
@@ -253,11 +254,11 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint
                 }
                 // a barrier between ranks keeps the adds to one element in rank order
                 __syncthreads();
-                // dense tiles (more than kBlock pairs of this rank): the rest, still in rank order
-                if (hi_s[r] > lo_s[r] + kBlock) {  // block-uniform
+                // dense tiles (more than kAccThreads pairs of this rank): the rest, still in rank order
+                if (hi_s[r] > lo_s[r] + kAccThreads) {  // block-uniform
                     const uint32_t lo = lo_s[r], hi = hi_s[r];
                     const uint32_t* pairs = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride) + 1;
-                    for (uint32_t p = lo + kBlock + threadIdx.x; p < hi; p += kBlock) {
+                    for (uint32_t p = lo + kAccThreads + threadIdx.x; p < hi; p += kAccThreads) {
                         const uint32_t o = pairs[2 * (uint64_t)p] - (uint32_t)tstart;
                         if (o < tlen) tile[o] = tile[o] + u2f(pairs[2 * (uint64_t)p + 1]);
                         else if (status) *status = MCCL_HIP_ERR_INDEX;
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint
     }
     float* out = acc + bstart + tstart;
     if (tlen == kAccTile && (((uintptr_t)out & 15) == 0)) {
-        for (int i = threadIdx.x; i < kAccTile / 4; i += kBlock) {
+        for (int i = threadIdx.x; i < kAccTile / 4; i += kAccThreads) {
             u4a v;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(kBlock) void k_sparse_accumulate_b(float* acc, uint
             __builtin_nontemporal_store(v, (u4a*)out + i);
         }
     } else {
-        for (uint32_t i = threadIdx.x; i < tlen; i += kBlock) {
+        for (uint32_t i = threadIdx.x; i < tlen; i += kAccThreads) {
             const float x = tile[i];
             out[i] = apply_scale ? x * scale : x;
         }
@@ -354,7 +355,7 @@ int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_ele
     const uint32_t bx = clamp_u32((kmax + kBlock * 8 - 1) / (kBlock * 8), 1, 0x7FFFFFFF);
     k_sparse_bounds<<<dim3(bx, (uint32_t)(nb * ws)), kBlock, 0, st>>>(wp, ws, wire_stride, n_total, bucket_elems,
                                                                         tiles, start, status);
-    k_sparse_accumulate_b<<<dim3(tiles, (uint32_t)nb), kBlock, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
+    k_sparse_accumulate_b<<<dim3(tiles, (uint32_t)nb), kAccThreads, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
                                                                          wire_stride, tiles, start, apply_scale,
                                                                          scale, status);
     return launch_status();
