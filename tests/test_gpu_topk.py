@@ -108,6 +108,22 @@ def test_single_pass_path_on_clustered_and_tied_inputs(ops):
     check_compress(ops, g, np.zeros(n, np.float32), 0.01)
     check_compress(ops, student_t(rng, n), (rng.standard_normal(n) * 1e-4).astype(np.float32), 0.001)
     check_compress(ops, student_t(rng, n), np.zeros(n, np.float32), 0.3, be=300_000)
+    # every sampled element (32-element runs, 5208 apart at this size) is 5.0 and nothing else is
+    # large: the candidate window sits at 5.0, the streaming pass stores 0.0 for all 12,288 of
+    # them, there are fewer candidates than k = 20,000, and the bucket falls back to the exact
+    # selection, which must see the values again
+    n = 2_000_000
+    g = student_t(rng, n, ties=0.0) * np.float32(1e-6)
+    for i in range(384):
+        g[5208 * i: 5208 * i + 32] = 5.0
+    check_compress(ops, g, np.zeros(n, np.float32), 0.01)
+    ws = ops.topk_workspace(n, n, 0.01, DEV)
+    try:
+        ops.set_tuning("topk_path", 2)
+        ops.topk_compress(to_dev(g, F32), to_dev(np.zeros(n, np.float32), F32), 0.01, workspace=ws)
+        assert ops.topk_path_report(ws, n, n, 0.01) == (0, 1)   # the scenario really takes the fallback
+    finally:
+        ops.set_tuning("topk_path", 0)
 
 
 def test_compress_many_buckets_short_last(ops):
