@@ -12,25 +12,31 @@
 //
 // FAST PATH (one pass over the gradient, 12 B/element of HBM traffic):
 //   sample     one block per bucket loads 12,288 evenly spread elements into
-//              LDS and radix-selects two of their keys: `lo`, which with 6 sigma
-//              of margin lies below the k-th largest key of the bucket, and
-//              `hi`, which with the same margin lies above it
-//   pass A     residual <- grad + residual in one streaming pass; elements with
-//              key >= lo ("candidates", about 1.7 k of them) are appended to
-//              per-bucket lists through per-wave LDS staging and counted in a
-//              256-bin histogram that is linear in the key over [lo, hi)
-//   select1    finds the histogram bin that holds the k-th largest key and
-//              copies that bin's candidates (a few hundred) to a second list
-//   select2    one block per bucket: checks that the lists are complete and
-//              the threshold lies inside the window (else the bucket is handed
-//              to the exact fallback), finishes the radix select on the second
-//              list: exact threshold key T, how many keys equal to T are taken
-//              and - when not all of them are - the largest index still taken
-//   mark       one block per candidate sub-list (= a fixed set of 8192-element
-//              tiles): pick bitmaps of its tiles in LDS, each pick's rank inside
-//              its tile by popcount prefix, picks written per tile in index
-//              order to a staging list, residual zeroed at the picks
-//   emit       concatenates the tiles' runs in tile order into the payload
+//              LDS and radix-selects three of their keys: `lo`, which with 6 sigma
+//              of margin lies below the k-th largest key of the bucket, `hi`,
+//              which with the same margin lies above it, and the predicted
+//              threshold itself
+//   pass A     residual <- grad + residual in one streaming pass, except that
+//              elements at or above the predicted threshold are stored as 0.0f
+//              at once; elements with key >= lo ("candidates", about 1.7 k) go,
+//              in index order, to the 64 slots of their region (the 2048
+//              elements one wavefront streams): no atomics, no shared lists.
+//              A region with more than 64 candidates is marked dense and later
+//              read from the residual itself
+//   hist       256-bin histogram of the candidates, linear in the key over [lo, hi)
+//   select1    finds the histogram bin that holds the k-th largest key, counts
+//              per region the candidates in higher bins (picks for certain) and
+//              copies the threshold bin's candidates (a few hundred) to list2
+//   select2    one block per bucket: checks that the threshold lies inside the
+//              window (else the bucket is handed to the exact fallback, after
+//              the pre-zeroed values have been put back), finishes the radix
+//              select on list2: exact threshold key T, how many keys equal to T
+//              are taken and - when not all of them are - the largest index still
+//              taken; adds list2's picks to the region counts and scans them
+//              into each region's offset in the payload
+//   emit       an ordered filter: a wavefront per region writes the region's
+//              picks at its offset and repairs the residual where the predicted
+//              threshold and T disagree (zero a missed pick, restore a non-pick)
 // EXACT PATH (any input; also the per-bucket fallback of the fast path):
 //   [pass A]   residual <- grad + residual, histogram of key[30:20]
 //   refine x2  histograms of key[19:10], key[9:0] among prefix matches
