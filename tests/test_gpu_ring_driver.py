@@ -65,6 +65,22 @@ def test_half_ring_rounds_every_step_like_the_wire(C, dt, chunked):
             _check_all_ranks(dts, dt, want)
 
 
+@pytest.mark.parametrize("dt", [F16, BF16])
+def test_half_ring_three_ranks_scale_in_fp32(C, dt):
+    # 1/3 is not exact in any format: the AVG tail multiplies by float(1/3) in fp32 and rounds once
+    ws = 3
+    g = C.LoopbackGroup(ws)
+    rng = np.random.default_rng(31 + dt)
+    inv = float(np.float32(1.0 / 3.0))
+    for n, chunked in ((70_001, True), (4099, False)):
+        ins = [rand_vals(rng, n, dt, sigma=1.0, specials=False) for _ in range(ws)]
+        want = oracle.ring_fold(ins, dt, OP_AVG, RING_CHUNKED if chunked else RING_BASIC, scale_by=inv, stepwise=True)
+        dts = [to_dev(x, dt) for x in ins]
+        g.allreduce_ring(dts, OP_AVG, chunked)
+        torch.cuda.synchronize()
+        _check_all_ranks(dts, dt, want)
+
+
 @pytest.mark.parametrize("n", [70_000, 70_001])
 @pytest.mark.parametrize("chunked", [False, True])
 def test_reference_three_rank_constants(C, n, chunked):
