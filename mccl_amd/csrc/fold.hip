@@ -160,8 +160,11 @@ __global__ __launch_bounds__(kBlock) void k_scale_int(T* buf, uint64_t n, float 
 }
 
 // ---- W-way fold in ring-step order --------------------------------------------
+// in[i] = buffer of rank i % ws for i < 2 * ws: the ws buffers in ring order
+// starting at any rank are ws consecutive entries, which a block fetches with
+// one wide scalar load instead of ws dependent ones.
 struct RingPtrs {
-    const void* in[MCCL_HIP_MAX_WORLD];
+    const void* in[2 * MCCL_HIP_MAX_WORLD];
 };
 
 // blockIdx.y = bucket * nchunks + chunk.  Each block row folds one chunk of one
@@ -198,6 +201,15 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
     u4a* ov = (u4a*)((char*)out + voff);
 
     const uint64_t tile = (uint64_t)kBlock * U;
+    const void* rp[WSC > 0 ? WSC : 1];  // rank buffers in fold order (compile-time world sizes)
+    if constexpr (WSC > 0) {
+#pragma unroll
+        for (int j = 0; j < WSC; j++) rp[j] = ptrs.in[first + j];
+    }
+    auto rank_ptr = [&](int j, int r) -> const char* {
+        if constexpr (WSC > 0) return (const char*)rp[j];
+        else return (const char*)ptrs.in[r];
+    };
     for (uint64_t base = (uint64_t)blockIdx.x * tile; base < nvec; base += (uint64_t)gridDim.x * tile) {
         if constexpr (DT == MCCL_HIP_F32) {
             float acc[U][4];
@@ -208,7 +220,7 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
                 if (idx[u] >= nvec) idx[u] = nvec - 1;  // clamp: recomputes a valid vector, store is guarded
             }
             {
-                const char* p = (const char*)ptrs.in[first] + voff;
+                const char* p = rank_ptr(0, first) + voff;
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     u4a v = load_vec_u<ES, NT>(p + idx[u] * 16);
@@ -220,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
 #pragma unroll
             for (int j = 1; j < ws; j++) {
                 r = (r + 1 == ws) ? 0 : r + 1;
-                const char* p = (const char*)ptrs.in[r] + voff;
+                const char* p = rank_ptr(j, r) + voff;
                 u4a v[U];
 #pragma unroll
                 for (int u = 0; u < U; u++) v[u] = load_vec_u<ES, NT>(p + idx[u] * 16);
@@ -245,7 +257,7 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
                 if (idx[u] >= nvec) idx[u] = nvec - 1;
             }
             {
-                const char* p = (const char*)ptrs.in[first] + voff;
+                const char* p = rank_ptr(0, first) + voff;
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     u4a v = load_vec_u<ES, NT>(p + idx[u] * 16);
@@ -260,7 +272,7 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
 #pragma unroll
             for (int j = 1; j < ws; j++) {
                 r = (r + 1 == ws) ? 0 : r + 1;
-                const char* p = (const char*)ptrs.in[r] + voff;
+                const char* p = rank_ptr(j, r) + voff;
                 u4a v[U];
 #pragma unroll
                 for (int u = 0; u < U; u++) v[u] = load_vec_u<ES, NT>(p + idx[u] * 16);
@@ -506,10 +518,11 @@ int mccl_hip_ring_fold(void* out, const void* const* host_in, int ws, uint64_t n
     if (c) return c < 0 ? c : MCCL_HIP_OK;
     if (bucket_elems == 0) return MCCL_HIP_ERR_ARG;
     RingPtrs ptrs;
-    for (int r = 0; r < MCCL_HIP_MAX_WORLD; r++) ptrs.in[r] = nullptr;
+    for (int r = 0; r < 2 * MCCL_HIP_MAX_WORLD; r++) ptrs.in[r] = nullptr;
     for (int r = 0; r < ws; r++) {
         if (!host_in[r]) return MCCL_HIP_ERR_ARG;
         ptrs.in[r] = host_in[r];
+        ptrs.in[ws + r] = host_in[r];
     }
     int rc = mccl_hip_init();
     if (rc) return rc;
