@@ -153,6 +153,21 @@ def test_config4_full_bucket_and_error_feedback_over_steps(ops):
     assert oracle.parse_wire(w)[0] == 65_536
 
 
+def test_one_large_bucket(ops):
+    # 20 M elements in one bucket: more regions than select2 keeps in registers (its generic sweep)
+    n = 20_000_003
+    rng = np.random.default_rng(99)
+    g = student_t(rng, n, ties=0.001)
+    res_o = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    dres = to_dev(res_o, F32)
+    ws = ops.topk_workspace(n, n, 0.01, DEV)
+    w, rc = oracle.topk_compress(g, res_o, 0.01)
+    wire, stride = ops.topk_compress(to_dev(g, F32), dres, 0.01, workspace=ws)
+    assert ops.topk_path_report(ws, n, n, 0.01) == (1, 1)
+    assert wire.cpu().numpy()[:rc].tobytes() == w.tobytes()
+    assert np.array_equal(bits(to_np(dres, F32)), bits(res_o))
+
+
 def test_compress_argument_errors(ops):
     from mccl_amd._lib import MCCLHipError
     g = torch.zeros(1000, device=DEV); r = torch.zeros(1000, device=DEV)
