@@ -243,6 +243,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def("allreduce_coalesced", [](mccl::LoopbackGroup& g, std::vector<std::vector<at::Tensor>> lists, int op) {
             g.allreduce_coalesced(lists, static_cast<c10d::ReduceOp::RedOpType>(op));
         }, py::arg("rank_lists"), py::arg("op") = 0)
+        .def("reduce_scatter", [](mccl::LoopbackGroup& g, std::vector<at::Tensor> outputs,
+                                  std::vector<std::vector<at::Tensor>> inputs, int op) {
+            g.reduce_scatter(outputs, inputs, static_cast<c10d::ReduceOp::RedOpType>(op));
+        }, py::arg("outputs"), py::arg("inputs"), py::arg("op") = 0)
         .def("allreduce_ring", [](mccl::LoopbackGroup& g, std::vector<at::Tensor> t, int op, bool chunked) {
             g.allreduce_ring(t, static_cast<c10d::ReduceOp::RedOpType>(op),
                              chunked ? mccl::RingAlgo::CHUNKED : mccl::RingAlgo::BASIC);

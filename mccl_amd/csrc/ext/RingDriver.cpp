@@ -193,6 +193,51 @@ void LoopbackGroup::allreduce_coalesced(std::vector<std::vector<at::Tensor>>& li
     }
 }
 
+void LoopbackGroup::reduce_scatter(std::vector<at::Tensor>& outputs, std::vector<std::vector<at::Tensor>>& inputs,
+                                   c10d::ReduceOp::RedOpType op) {
+    MCCL_CHECK_TENSOR(static_cast<int>(outputs.size()) == ws_ && static_cast<int>(inputs.size()) == ws_,
+                      "one output and one input list per rank expected");
+    for (int r = 0; r < ws_; r++) {
+        MCCL_CHECK_TENSOR(static_cast<int>(inputs[r].size()) == ws_, "Input tensor list size must equal world_size");
+        check_single_tensor(outputs[r]);
+        for (auto& x : inputs[r]) {
+            MCCL_CHECK_TENSOR(x.is_contiguous(), "MCCL v1 requires contiguous tensors. Call .contiguous() before passing to collective.");
+            check_single_tensor(x);
+            check_same_shape_dtype(outputs[r], x);
+        }
+        check_same_shape_dtype(outputs[0], outputs[r]);
+    }
+    if (outputs[0].numel() == 0) return;
+    metal_kernels_init();
+    if (ws_ == 1) {
+        outputs[0].copy_(inputs[0][0]);
+    } else if (ws_ == 2) {
+        // step 0 of the ring: rank r sends chunk (r + 1) % 2 and folds the incoming
+        // partial into its own chunk r; both folds read the peer's untouched chunk
+        for (int r = 0; r < 2; r++) {
+            metal_reduce_op_fenced(inputs[r][r], inputs[1 - r][r], op);
+            stats_.reduce_launches++;
+            stats_.fences_signalled++;
+            stats_.wire_bytes += tensor_nbytes(outputs[r]);
+        }
+        for (int r = 0; r < 2; r++) outputs[r].copy_(inputs[r][r]);
+        stats_.copy_launches += 2;
+    } else {
+        for (int d = 0; d < ws_; d++) {
+            outputs[d].copy_(inputs[d][d]);
+            stats_.copy_launches++;
+            for (int src = 0; src < ws_; src++) {
+                if (src == d) continue;
+                metal_reduce_op(outputs[d], inputs[src][d], op);
+                stats_.reduce_launches++;
+                stats_.wire_bytes += tensor_nbytes(outputs[d]);
+            }
+        }
+    }
+    stats_.collectives++;
+    stats_.last_algo = ws_ >= 3 ? "reduce_scatter_star" : "reduce_scatter_ring";
+}
+
 // What `from_rank`'s tensor looks like on the far side of the link: compressed
 // with the sender's state and expanded again, or the bytes themselves.
 at::Tensor LoopbackGroup::through_wire(int from_rank, const at::Tensor& tensor) {

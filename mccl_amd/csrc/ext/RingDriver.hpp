@@ -99,6 +99,15 @@ public:
     /// Flatten, one allreduce, scatter back (csrc/backend/ProcessGroupMCCL.cpp:1381-1468).
     void allreduce_coalesced(std::vector<std::vector<at::Tensor>>& rank_lists, c10d::ReduceOp::RedOpType op);
 
+    /// outputs[d] = fold over ranks of inputs[rank][d]
+    /// (csrc/backend/ProcessGroupMCCL.cpp:3133-3313): with three or more ranks the
+    /// star form, rank d's own contribution first and the others in ascending
+    /// rank order (:2764-2815); with two ranks one ring step that folds into the
+    /// input chunk in place (:3257-3301).  AVG adds and does not scale: the
+    /// reference's reduce_scatter never multiplies by 1/ws.
+    void reduce_scatter(std::vector<at::Tensor>& outputs, std::vector<std::vector<at::Tensor>>& inputs,
+                        c10d::ReduceOp::RedOpType op);
+
     void allreduce_ring(std::vector<at::Tensor>& rank_tensors, c10d::ReduceOp::RedOpType op, RingAlgo algo);
     void allreduce_two_rank(std::vector<at::Tensor>& rank_tensors, c10d::ReduceOp::RedOpType op);
     void allreduce_small(std::vector<at::Tensor>& rank_tensors, c10d::ReduceOp::RedOpType op);

@@ -256,6 +256,31 @@ def test_coalesced_flattens_and_scatters(C):
         g.allreduce_coalesced([[], [], []], OP_SUM)
 
 
+@pytest.mark.parametrize("ws", [1, 2, 3, 5])
+def test_reduce_scatter_order_and_no_avg_scale(C, ws):
+    # own contribution first, the others in ascending rank order; AVG adds without scaling
+    g = C.LoopbackGroup(ws)
+    rng = np.random.default_rng(40 + ws)
+    n = 70_001
+    for op in (OP_SUM, OP_AVG, OP_MAX):
+        host = [[rand_vals(rng, n, F32, sigma=1e-3, specials=False) for _ in range(ws)] for _ in range(ws)]
+        ins = [[to_dev(x, F32) for x in row] for row in host]
+        outs = [torch.empty(n, device=DEV) for _ in range(ws)]
+        g.reduce_scatter(outs, ins, op)
+        torch.cuda.synchronize()
+        for d in range(ws):
+            want = host[d][d].copy()
+            for src in range(ws):
+                if src != d:
+                    oracle.fold2(want, host[src][d], F32, OP_SUM if op == OP_AVG else op)
+            assert np.array_equal(bits(to_np(outs[d], F32)), bits(want)), (op, d)
+    if ws > 1:
+        assert g.stats()["last_algo"] == ("reduce_scatter_star" if ws >= 3 else "reduce_scatter_ring")
+    with pytest.raises(RuntimeError, match="Input tensor list size must equal world_size"):
+        g.reduce_scatter([torch.empty(4, device=DEV) for _ in range(ws)],
+                         [[torch.empty(4, device=DEV)] * (ws + 1) for _ in range(ws)], OP_SUM)
+
+
 def test_argument_checks(C):
     g = C.LoopbackGroup(3)
     with pytest.raises(RuntimeError, match="one tensor per rank expected"):
