@@ -84,6 +84,7 @@ def main() -> int:
         return nbytes / (ms * 1e-3) / 1e9
 
     extra = {}
+    roofline_topk = None
 
     # ---- config 2: the headline workload -----------------------------------
     gens = [torch.Generator(device=dev).manual_seed(1000 + r) for r in range(W)]
@@ -197,6 +198,14 @@ def main() -> int:
                                           "elems_per_s": N / (tk["avg_ms"] * 1e-3),
                                           "bytes": topk_bytes, "buckets": nb, "k_per_bucket": ks[0],
                                           "single_pass_buckets": ops.topk_path_report(wsb, N, BUCKET, 0.01)[0]}
+        # second half of the headline metric: same fields as `roofline`, for the whole
+        # compress call (six launches); traffic from the FETCH_SIZE / WRITE_SIZE counter
+        # runs in profiles/topk_and_sparse_accumulate_hbm_traffic.md (default workload only)
+        roofline_topk = {"bound": "hbm", "kernel": "mccl_hip_topk_compress (6 launches, dominant k_topk_pass_a_fast)",
+                         "achieved": rate(topk_bytes, tk["avg_ms"]), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": rate(topk_bytes, tk["avg_ms"]) / HBM_PEAK_GBPS,
+                         "traffic": 1_236_252_262 if N == N_GRAD else None,
+                         "bytes_per_launch": topk_bytes, "avg_launch_ms": tk["avg_ms"], "min_launch_ms": tk["min_ms"]}
         # one bucket alone (the reference's call granularity; cache resident)
         r1 = residual0[:BUCKET].clone()
         ws1 = ops.topk_workspace(BUCKET, BUCKET, 0.01, dev)
@@ -311,6 +320,7 @@ def main() -> int:
                    "elements": N, "world_size": W, "bucket_elems": BUCKET, "bytes_per_element": 36,
                    "elements_per_s": N / (wall_ms * 1e-3), "pct_of_hbm_peak": 100.0 * fold_gbps / HBM_PEAK_GBPS},
         "roofline": roofline,
+        "roofline_topk": roofline_topk,
         "cpu_baseline": cpu,
         "extra": extra,
     }
