@@ -94,14 +94,17 @@ struct ElemInfo {
 };
 
 // ---- wave / block prefix sums ----------------------------------------------
-// Inclusive scan of `v` across the 64 lanes of a wavefront.
+// Inclusive scan of `v` across the 64 lanes of a wavefront, on the DPP data path
+// (no LDS traffic): shifts by 1, 2, 4, 8 inside each row of 16 lanes, then lane
+// 15 of rows 0 and 2 is added to rows 1 and 3, then lane 31 to rows 2 and 3.
+// Lanes without a source, and rows masked out, read the `old` operand, 0.
 __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
-    const int lane = threadIdx.x & (kWave - 1);
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        uint32_t t = __shfl_up(v, d, kWave);
-        if (lane >= d) v += t;
-    }
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, true);   // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, true);   // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, true);   // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, true);   // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xA, 0xF, false);  // row_bcast:15 -> rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, false);  // row_bcast:31 -> rows 2, 3
     return v;
 }
 
