@@ -51,21 +51,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     py::class_<mccl::MCCLOptions, c10d::Backend::Options, c10::intrusive_ptr<mccl::MCCLOptions>>(m, "MCCLOptions")
         .def(py::init<>())
         .def(py::init<std::chrono::milliseconds>(), py::arg("timeout"))
-        .def_readwrite("transport", &mccl::MCCLOptions::transport)
-        .def_readwrite("listen_addr", &mccl::MCCLOptions::listen_addr)
-        .def_readwrite("port_base", &mccl::MCCLOptions::port_base)
-        .def_readwrite("ifname", &mccl::MCCLOptions::ifname)
-        .def_readwrite("chunk_bytes", &mccl::MCCLOptions::chunk_bytes)
-        .def_readwrite("small_msg_threshold", &mccl::MCCLOptions::small_msg_threshold)
-        .def_readwrite("transport_crc", &mccl::MCCLOptions::transport_crc)
-        .def_readwrite("fast_math", &mccl::MCCLOptions::fast_math)
-        .def_readwrite("gpu_threshold", &mccl::MCCLOptions::gpu_threshold)
-        .def_readwrite("overlap_comm", &mccl::MCCLOptions::overlap_comm)
-        .def_readwrite("max_queue_depth", &mccl::MCCLOptions::max_queue_depth)
-        .def_readwrite("compression", &mccl::MCCLOptions::compression)
-        .def_readwrite("topk_ratio", &mccl::MCCLOptions::topk_ratio)
-        .def_readwrite("watchdog_timeout", &mccl::MCCLOptions::watchdog_timeout)
-        .def_readwrite("heartbeat_interval", &mccl::MCCLOptions::heartbeat_interval);
+#define MCCL_OPTION_PROPERTY(type, name, init) .def_readwrite(#name, &mccl::MCCLOptions::name)
+        MCCL_OPTION_TABLE(MCCL_OPTION_PROPERTY);
+#undef MCCL_OPTION_PROPERTY
 
     // ---- kernel helpers: same names as the reference's test bindings ----------
     m.def("_metal_accumulate_chunk", [](at::Tensor dst, const at::Tensor& src) {
