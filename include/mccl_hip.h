@@ -40,6 +40,7 @@ extern "C" {
 #define MCCL_HIP_ERR_RUNTIME (-7)   /* a HIP runtime call failed; see mccl_hip_last_hip_error()     */
 #define MCCL_HIP_ERR_WORKSPACE (-8) /* workspace smaller than mccl_hip_topk_workspace_bytes()       */
 #define MCCL_HIP_ERR_TIMEOUT (-9)   /* fence wait exceeded its limit (csrc/metal/EventSync.mm:37-71) */
+#define MCCL_HIP_ERR_POINTER (-10)  /* the bytes are not memory a kernel on the current GPU can reach */
 
 /* ---- element types (at::ScalarType values) ------------------------------ */
 #define MCCL_HIP_U8 0
@@ -79,6 +80,16 @@ int mccl_hip_abi_version(void);
 const char* mccl_hip_strerror(int code);
 /* hipError_t value of the most recent failing runtime call on this thread. */
 int mccl_hip_last_hip_error(void);
+
+/* The reference's raw-pointer folds (csrc/metal/AccelerateOps.hpp:18-59) run
+ * on CPU-visible memory that the GPU shares.  Their counterparts here launch
+ * kernels, so a caller holding a raw pointer first asks whether a kernel on the
+ * current device can reach [ptr, ptr + nbytes): device memory of the current
+ * GPU (the range must lie inside one allocation), managed memory, or pinned
+ * host memory.  On success *device_ptr receives the address to hand to the
+ * kernels (for pinned host memory its device-side alias).  Pageable host memory
+ * and foreign pointers give MCCL_HIP_ERR_POINTER; nothing is launched. */
+int mccl_hip_pointer_check(const void* ptr, uint64_t nbytes, void** device_ptr);
 
 /* ---- binary folds: one ring step ---------------------------------------- */
 
@@ -185,7 +196,7 @@ int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_ele
                                int apply_scale, float scale, int* status, void* workspace,
                                uint64_t workspace_bytes, void* stream);
 /* Scratch for mccl_hip_sparse_accumulate (per rank and bucket, the position in
- * the payload at which every 4096-element output tile begins).  Passing
+ * the payload at which every 8192-element output tile begins).  Passing
  * workspace = NULL is allowed: the ranges are then found by binary search in
  * every block, which costs about 3x the time on MI355X. */
 uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, int ws);
@@ -203,12 +214,18 @@ int mccl_hip_cast_f16_to_f32(const void* src, float* dst, uint64_t n, void* stre
 
 /* Replaces next_fence_event_value() + signal_mccl_fence_gpu()
  * (csrc/metal/EventSync.mm:189-200): records an event on `stream` and returns
- * its ticket (monotonic, never 0) in *ticket. */
+ * its ticket (monotonic, never 0) in *ticket.  A ticket covers the work
+ * enqueued on ITS stream before the signal.  (The reference's shared-event
+ * values are signalled from one queue, so there "value v reached" implies every
+ * smaller value; here that holds per stream: wait on the last ticket of every
+ * stream whose work matters.)  The library keeps the newest 1024 tickets'
+ * events; a signal that pushes an older ticket out first waits, on the host,
+ * until that ticket's work has completed, so a ticket that is no longer held is
+ * always complete. */
 int mccl_hip_fence_signal(void* stream, uint64_t* ticket);
 /* Replaces wait_for_mccl_fence() (EventSync.mm:202-206): blocks the host until
- * everything enqueued before the ticket has completed.  timeout_ms <= 0 uses
- * the reference's 30 s limit.  Tickets older than the event ring are complete
- * by construction. */
+ * everything enqueued on the ticket's stream before the signal has completed.
+ * timeout_ms <= 0 uses the reference's 30 s limit. */
 int mccl_hip_fence_wait(uint64_t ticket, int timeout_ms);
 /* Non-blocking: 1 complete, 0 pending, negative on error. */
 int mccl_hip_fence_query(uint64_t ticket);

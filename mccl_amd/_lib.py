@@ -18,6 +18,7 @@ SIGNATURES = {
     "mccl_hip_abi_version": (_i32, []),
     "mccl_hip_strerror": (C.c_char_p, [_i32]),
     "mccl_hip_last_hip_error": (_i32, []),
+    "mccl_hip_pointer_check": (_i32, [_vp, _u64, C.POINTER(_vp)]),
     "mccl_hip_fold2": (_i32, [_vp, _vp, _u64, _i32, _i32, _vp]),
     "mccl_hip_scale": (_i32, [_vp, _u64, _i32, _f32, _vp]),
     "mccl_hip_fold2_scale": (_i32, [_vp, _vp, _u64, _i32, _f32, _vp]),

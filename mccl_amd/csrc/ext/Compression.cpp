@@ -135,10 +135,6 @@ void TopKCompressor::decompress(const void* src, size_t compressed_size, void* d
     if (st == MCCL_HIP_ERR_INDEX) throw MCCLError("TopK decompress: index out of bounds");
 }
 
-std::string TopKCompressor::name() const { return "topk"; }
-std::string FP16Compressor::name() const { return "fp16"; }
-size_t FP16Compressor::max_compressed_size(size_t nbytes) const { return nbytes; }  // FP16Compression.cpp:165-168
-
 size_t TopKCompressor::max_compressed_size(size_t nbytes) const {
     return static_cast<size_t>(mccl_hip_topk_max_compressed_size(nbytes, k_ratio_));
 }

@@ -19,25 +19,22 @@ enum class CompressionMode : int {
     TOPK = 2,
 };
 
-// The four members of the interface, spelled once: MCCL_COMPRESSOR_MEMBERS(virtual, = 0)
-// declares them in the base class, MCCL_COMPRESSOR_MEMBERS(, override) in an
-// implementation.
-//   compress    nbytes at src -> payload at dst (capacity dst_capacity); returns the payload
-//               size.  stable_id names the logical tensor across steps; stateful
-//               compressors key their residual on it.
-//   decompress  compressed_size bytes at src -> nbytes at dst
-#define MCCL_COMPRESSOR_MEMBERS(pre, post)                                                              \
-    pre size_t compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,                 \
-                        at::ScalarType dtype, uint64_t stable_id = 0) post;                             \
-    pre void decompress(const void* src, size_t compressed_size, void* dst, size_t nbytes,              \
-                        at::ScalarType dtype) post;                                                     \
-    pre size_t max_compressed_size(size_t nbytes) const post;                                           \
-    pre std::string name() const post;
-
 class Compressor {
 public:
     virtual ~Compressor() = default;
-    MCCL_COMPRESSOR_MEMBERS(virtual, = 0)
+
+    /// Compresses nbytes at src into dst (capacity dst_capacity); returns the
+    /// payload size.  stable_id names the logical tensor across steps; stateful
+    /// compressors key their residual on it.
+    virtual size_t compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
+                            at::ScalarType dtype, uint64_t stable_id = 0) = 0;
+
+    /// Expands compressed_size bytes at src into nbytes at dst.
+    virtual void decompress(const void* src, size_t compressed_size, void* dst, size_t nbytes,
+                            at::ScalarType dtype) = 0;
+
+    virtual size_t max_compressed_size(size_t nbytes) const = 0;
+    virtual std::string name() const = 0;
 };
 
 /// NONE -> nullptr, FP16 -> FP16Compressor, TOPK -> TopKCompressor(param > 0 ?

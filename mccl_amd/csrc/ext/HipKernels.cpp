@@ -27,6 +27,11 @@ std::atomic<bool> g_initialized{false};
 
 void* current_stream(int device) { return c10::hip::getCurrentHIPStream(device).stream(); }
 
+bool op_is_unsupported(c10d::ReduceOp::RedOpType op) {
+    return !(op == c10d::ReduceOp::SUM || op == c10d::ReduceOp::AVG || op == c10d::ReduceOp::MIN ||
+             op == c10d::ReduceOp::MAX || op == c10d::ReduceOp::PRODUCT);
+}
+
 int64_t safe_numel(const at::Tensor& t) {
     const int64_t n = t.numel();
     MCCL_CHECK(n >= 0 && static_cast<uint64_t>(n) <= MCCL_HIP_MAX_ELEMS,
@@ -216,28 +221,59 @@ void wait_for_mccl_fence(uint64_t value) {
 }
 
 // ---- raw-pointer folds --------------------------------------------------------
+// The reference calls this family with view.cpu_ptr, memory the CPU and the GPU
+// share (csrc/backend/ProcessGroupMCCL.cpp:494-498).  Here the arithmetic runs in
+// a kernel, so every pointer is first resolved to an address a kernel can use:
+// device memory of the current GPU, managed memory, or pinned host memory (its
+// device-side alias).  Anything else, pageable host memory above all, throws
+// before a kernel is launched; there is no host fallback.
 namespace {
+size_t elem_bytes(int dtype) {
+    switch (dtype) {
+        case MCCL_HIP_F32: case MCCL_HIP_I32: return 4;
+        case MCCL_HIP_F16: case MCCL_HIP_BF16: return 2;
+        case MCCL_HIP_I64: return 8;
+        default: return 1;
+    }
+}
+void* kernel_pointer(const void* p, int64_t n, int dtype, const char* what) {
+    MCCL_CHECK(n >= 0 && static_cast<uint64_t>(n) <= MCCL_HIP_MAX_ELEMS,
+               std::string(what) + ": element count out of range");
+    if (n == 0) return const_cast<void*>(p);
+    void* dp = nullptr;
+    const int rc = mccl_hip_pointer_check(p, static_cast<uint64_t>(n) * elem_bytes(dtype), &dp);
+    if (rc == MCCL_HIP_ERR_POINTER || rc == MCCL_HIP_ERR_ARG)
+        throw TensorError(std::string(what) + ": the buffer is not memory a GPU kernel can reach (device, managed "
+                          "or pinned host memory of the current device is required; pageable host memory is "
+                          "not accepted and there is no host fallback)");
+    throw_on_status(rc, what);
+    return dp;
+}
 void raw_fold(void* dst, const void* src, int64_t n, int dtype, c10d::ReduceOp::RedOpType op,
               const char* what) {
     metal_kernels_init();
-    void* st = c10::hip::getCurrentHIPStream().stream();
-    int rc = mccl_hip_fold2(dst, src, static_cast<uint64_t>(n), dtype, static_cast<int>(op), st);
-    if (rc == MCCL_HIP_ERR_OP)
+    if (op_is_unsupported(op))
         throw MCCLError(std::string("Unsupported ReduceOp for ") + what + ": " +
                         std::to_string(static_cast<int>(op)));
-    throw_on_status(rc, what);
+    void* d = kernel_pointer(dst, n, dtype, what);
+    const void* s = kernel_pointer(src, n, dtype, what);
+    void* st = c10::hip::getCurrentHIPStream().stream();
+    throw_on_status(mccl_hip_fold2(d, s, static_cast<uint64_t>(n), dtype, static_cast<int>(op), st), what);
     throw_on_status(mccl_hip_sync(st), what);
 }
 void raw_scale(void* buf, int64_t n, int dtype, float scale) {
     metal_kernels_init();
+    void* b = kernel_pointer(buf, n, dtype, "scale");
     void* st = c10::hip::getCurrentHIPStream().stream();
-    throw_on_status(mccl_hip_scale(buf, static_cast<uint64_t>(n), dtype, scale, st), "scale");
+    throw_on_status(mccl_hip_scale(b, static_cast<uint64_t>(n), dtype, scale, st), "scale");
     throw_on_status(mccl_hip_sync(st), "scale");
 }
 void raw_fused(void* dst, const void* src, int64_t n, int dtype, float scale) {
     metal_kernels_init();
+    void* d = kernel_pointer(dst, n, dtype, "fused");
+    const void* s = kernel_pointer(src, n, dtype, "fused");
     void* st = c10::hip::getCurrentHIPStream().stream();
-    throw_on_status(mccl_hip_fold2_scale(dst, src, static_cast<uint64_t>(n), dtype, scale, st), "fused");
+    throw_on_status(mccl_hip_fold2_scale(d, s, static_cast<uint64_t>(n), dtype, scale, st), "fused");
     throw_on_status(mccl_hip_sync(st), "fused");
 }
 int integral_code(at::ScalarType t, const char* fn) {

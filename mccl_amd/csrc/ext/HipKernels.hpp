@@ -48,8 +48,11 @@ void signal_mccl_fence_gpu(uint64_t value);
 void wait_for_mccl_fence(uint64_t value);
 
 // ---- raw-pointer folds (csrc/metal/AccelerateOps.hpp:18-59) -----------------
-// Same names and argument order; the pointers are DEVICE pointers here and the
-// calls return after the work has completed, like the reference's host folds.
+// Same names and argument order.  The reference hands these memory that CPU and
+// GPU share; here the pointers must be memory a kernel on the current device can
+// reach (device, managed or pinned host memory): each call checks that first and
+// throws TensorError otherwise, before anything is launched.  The calls return
+// after the work has completed, like the reference's host folds.
 void cpu_accumulate(float* dst, const float* src, int64_t count);
 void cpu_scale_inplace(float* buf, int64_t count, float scale);
 void cpu_accumulate_and_scale(float* dst, const float* src, int64_t count, float scale);

@@ -29,6 +29,30 @@ namespace {
 // helpers stay blocking calls.
 void producer_sync() { mccl::metal_sync(); }
 
+// Argument checks of the raw-pointer test bindings: the tensors only lend their
+// data pointers, so they may be GPU tensors or (pinned) host tensors.
+void raw_check(const at::Tensor& dst, const at::Tensor* src, c10::optional<at::ScalarType> only = c10::nullopt) {
+    MCCL_CHECK_TENSOR(dst.is_contiguous(), "MCCL v1 requires contiguous tensors. Call .contiguous() before passing "
+                                           "to collective.");
+    if (src) {
+        mccl::check_same_shape_dtype(dst, *src);
+        MCCL_CHECK_TENSOR(src->is_contiguous(), "MCCL v1 requires contiguous tensors. Call .contiguous() before "
+                                                "passing to collective.");
+    }
+    if (only) MCCL_CHECK(dst.scalar_type() == *only, "float32 only");
+}
+
+// A compressed payload handed to decompress: uint8, contiguous, on the GPU, and
+// at least as long as the size the caller says arrived.
+void check_payload(const at::Tensor& wire, const py::object& size, int64_t numel) {
+    mccl::check_single_tensor(wire);
+    MCCL_CHECK_TENSOR(wire.scalar_type() == at::kByte, "compressed payload must be a uint8 tensor");
+    MCCL_CHECK(numel >= 0, "decompress: negative element count");
+    if (!size.is_none())
+        MCCL_CHECK(size.cast<size_t>() <= static_cast<size_t>(wire.numel()),
+                   "decompress: compressed_size exceeds the payload tensor");
+}
+
 uint64_t stable_id_of(const at::Tensor& t) {
     // storage address + offset, stable across steps for DDP buckets
     // (csrc/backend/ProcessGroupMCCL.cpp:1080-1083)
@@ -51,9 +75,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     py::class_<mccl::MCCLOptions, c10d::Backend::Options, c10::intrusive_ptr<mccl::MCCLOptions>>(m, "MCCLOptions")
         .def(py::init<>())
         .def(py::init<std::chrono::milliseconds>(), py::arg("timeout"))
-#define MCCL_OPTION_PROPERTY(type, name, init) .def_readwrite(#name, &mccl::MCCLOptions::name)
-        MCCL_OPTION_TABLE(MCCL_OPTION_PROPERTY);
-#undef MCCL_OPTION_PROPERTY
+        .def_readwrite("transport", &mccl::MCCLOptions::transport)
+        .def_readwrite("listen_addr", &mccl::MCCLOptions::listen_addr)
+        .def_readwrite("port_base", &mccl::MCCLOptions::port_base)
+        .def_readwrite("ifname", &mccl::MCCLOptions::ifname)
+        .def_readwrite("chunk_bytes", &mccl::MCCLOptions::chunk_bytes)
+        .def_readwrite("small_msg_threshold", &mccl::MCCLOptions::small_msg_threshold)
+        .def_readwrite("transport_crc", &mccl::MCCLOptions::transport_crc)
+        .def_readwrite("fast_math", &mccl::MCCLOptions::fast_math)
+        .def_readwrite("gpu_threshold", &mccl::MCCLOptions::gpu_threshold)
+        .def_readwrite("overlap_comm", &mccl::MCCLOptions::overlap_comm)
+        .def_readwrite("max_queue_depth", &mccl::MCCLOptions::max_queue_depth)
+        .def_readwrite("compression", &mccl::MCCLOptions::compression)
+        .def_readwrite("topk_ratio", &mccl::MCCLOptions::topk_ratio)
+        .def_readwrite("watchdog_timeout", &mccl::MCCLOptions::watchdog_timeout)
+        .def_readwrite("heartbeat_interval", &mccl::MCCLOptions::heartbeat_interval);
 
     // ---- kernel helpers: same names as the reference's test bindings ----------
     m.def("_metal_accumulate_chunk", [](at::Tensor dst, const at::Tensor& src) {
@@ -113,14 +149,75 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return out;
     }, py::arg("out"), py::arg("ins"), py::arg("op"), py::arg("chunked") = false,
        py::arg("bucket_elems") = 0, py::arg("stepwise") = false);
+    // ---- raw-pointer family (csrc/metal/AccelerateOps.hpp:18-59) on tensors' data pointers.
+    // Tensors may live on the GPU or in pinned host memory; the functions themselves
+    // refuse memory a kernel cannot reach.  The *_ptr forms take plain addresses.
     m.def("_cpu_reduce_op", [](at::Tensor dst, const at::Tensor& src, int op) {
-        // raw-pointer family on device pointers, fp32 only here (test hook)
-        mccl::check_same_shape_dtype(dst, src);
-        MCCL_CHECK(dst.scalar_type() == at::kFloat, "float32 only");
-        mccl::cpu_reduce_op(dst.data_ptr<float>(), src.data_ptr<float>(), dst.numel(),
-                            static_cast<c10d::ReduceOp::RedOpType>(op));
+        raw_check(dst, &src);
+        const auto rop = static_cast<c10d::ReduceOp::RedOpType>(op);
+        const int64_t n = dst.numel();
+        switch (dst.scalar_type()) {
+            case at::kFloat: mccl::cpu_reduce_op(dst.data_ptr<float>(), src.data_ptr<float>(), n, rop); break;
+            case at::kHalf: mccl::cpu_reduce_op_half(dst.data_ptr<c10::Half>(), src.data_ptr<c10::Half>(), n, rop); break;
+            case at::kBFloat16:
+                mccl::cpu_reduce_op_bf16(dst.data_ptr<c10::BFloat16>(), src.data_ptr<c10::BFloat16>(), n, rop);
+                break;
+            default: mccl::cpu_reduce_op_integral(dst.data_ptr(), src.data_ptr(), n, dst.scalar_type(), rop);
+        }
         return dst;
     });
+    m.def("_cpu_scale_inplace", [](at::Tensor buf, double scale) {
+        raw_check(buf, nullptr);
+        const int64_t n = buf.numel();
+        const float s = static_cast<float>(scale);
+        switch (buf.scalar_type()) {
+            case at::kFloat: mccl::cpu_scale_inplace(buf.data_ptr<float>(), n, s); break;
+            case at::kHalf: mccl::cpu_scale_inplace_half(buf.data_ptr<c10::Half>(), n, s); break;
+            case at::kBFloat16: mccl::cpu_scale_inplace_bf16(buf.data_ptr<c10::BFloat16>(), n, s); break;
+            default: mccl::cpu_scale_inplace_integral(buf.data_ptr(), n, buf.scalar_type(), s);
+        }
+        return buf;
+    });
+    m.def("_cpu_accumulate_and_scale", [](at::Tensor dst, const at::Tensor& src, double scale) {
+        raw_check(dst, &src);
+        const int64_t n = dst.numel();
+        const float s = static_cast<float>(scale);
+        switch (dst.scalar_type()) {
+            case at::kFloat: mccl::cpu_accumulate_and_scale(dst.data_ptr<float>(), src.data_ptr<float>(), n, s); break;
+            case at::kHalf:
+                mccl::cpu_accumulate_and_scale_half(dst.data_ptr<c10::Half>(), src.data_ptr<c10::Half>(), n, s);
+                break;
+            case at::kBFloat16:
+                mccl::cpu_accumulate_and_scale_bf16(dst.data_ptr<c10::BFloat16>(), src.data_ptr<c10::BFloat16>(), n, s);
+                break;
+            default: throw mccl::MCCLError("cpu_accumulate_and_scale: float32/float16/bfloat16 only");
+        }
+        return dst;
+    });
+    m.def("_cpu_accumulate", [](at::Tensor dst, const at::Tensor& src) {
+        raw_check(dst, &src, at::kFloat);
+        mccl::cpu_accumulate(dst.data_ptr<float>(), src.data_ptr<float>(), dst.numel());
+        return dst;
+    });
+    m.def("_cpu_elementwise_min", [](at::Tensor dst, const at::Tensor& src) {
+        raw_check(dst, &src, at::kFloat);
+        mccl::cpu_elementwise_min(dst.data_ptr<float>(), src.data_ptr<float>(), dst.numel());
+        return dst;
+    });
+    m.def("_cpu_elementwise_max", [](at::Tensor dst, const at::Tensor& src) {
+        raw_check(dst, &src, at::kFloat);
+        mccl::cpu_elementwise_max(dst.data_ptr<float>(), src.data_ptr<float>(), dst.numel());
+        return dst;
+    });
+    m.def("_cpu_elementwise_product", [](at::Tensor dst, const at::Tensor& src) {
+        raw_check(dst, &src, at::kFloat);
+        mccl::cpu_elementwise_product(dst.data_ptr<float>(), src.data_ptr<float>(), dst.numel());
+        return dst;
+    });
+    m.def("_cpu_reduce_op_ptr", [](uint64_t dst, uint64_t src, int64_t count, int op) {
+        mccl::cpu_reduce_op(reinterpret_cast<float*>(dst), reinterpret_cast<const float*>(src), count,
+                            static_cast<c10d::ReduceOp::RedOpType>(op));
+    }, "cpu_reduce_op on two raw addresses of `count` floats");
 
     // ---- compressor -------------------------------------------------------------
     py::class_<mccl::Compressor>(m, "Compressor");
@@ -140,6 +237,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         }, py::arg("tensor"), py::arg("stable_id") = py::none(), py::arg("capacity") = py::none(),
            "Top-k payload of a gradient bucket as a uint8 device tensor; error feedback is kept per stable_id")
         .def("decompress", [](mccl::TopKCompressor& c, const at::Tensor& wire, int64_t numel, py::object size) {
+            check_payload(wire, size, numel);
             at::Tensor out = at::empty({numel}, at::TensorOptions().dtype(at::kFloat).device(wire.device()));
             const size_t sz = size.is_none() ? static_cast<size_t>(wire.numel()) : size.cast<size_t>();
             c.decompress(wire.data_ptr(), sz, out.data_ptr(), static_cast<size_t>(numel) * 4, at::kFloat);
@@ -169,6 +267,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
            "Half-precision payload of a float32 bucket (a float16 bucket is copied) as a uint8 device tensor")
         .def("decompress", [](mccl::FP16Compressor& c, const at::Tensor& wire, int64_t numel, py::object size,
                               at::ScalarType dtype) {
+            check_payload(wire, size, numel);
             at::Tensor out = at::empty({numel}, at::TensorOptions().dtype(dtype).device(wire.device()));
             const size_t sz = size.is_none() ? static_cast<size_t>(wire.numel()) : size.cast<size_t>();
             c.decompress(wire.data_ptr(), sz, out.data_ptr(), static_cast<size_t>(numel) * out.element_size(), dtype);

@@ -108,6 +108,9 @@ void compressed_unpack(Compressor* compressor, const CompressedFrame& frame, con
     MCCL_CHECK(frame.wire_size > 0 && frame.wire_size <= max_comp,
                "Compressed payload size " + std::to_string(frame.wire_size) + " out of range (max " +
                    std::to_string(max_comp) + ")");
+    MCCL_CHECK_TENSOR(frame.payload.defined() && frame.payload.is_cuda() &&
+                          frame.payload.get_device() == out.get_device(),
+                      "compressed payload must live on the output tensor's GPU");
     MCCL_CHECK(frame.payload.defined() && frame.payload.scalar_type() == at::kByte && frame.payload.is_contiguous() &&
                    static_cast<uint64_t>(frame.payload.numel()) == frame.wire_size,
                "compressed_recv recv_chunks failed");

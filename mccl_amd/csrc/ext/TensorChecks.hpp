@@ -17,42 +17,26 @@
 
 namespace mccl {
 
-namespace detail {
-// Element types a collective accepts: the training types, the metadata types and float64.
-inline bool accepted_dtype(at::ScalarType dt) {
-    constexpr at::ScalarType kAccepted[] = {at::kFloat, at::kHalf, at::kBFloat16, at::kLong,
-                                            at::kInt,   at::kBool, at::kByte,     at::kDouble};
-    for (at::ScalarType a : kAccepted)
-        if (a == dt) return true;
-    return false;
-}
-}  // namespace detail
-
-// Empty tensors pass: collectives treat them as no-ops.
 inline void check_single_tensor(const at::Tensor& t) {
-    if (!t.is_cuda())
-        detail::fail<TensorError>("Tensor check failed: ", "t.is_cuda()", nullptr, 0,
-                                  "MCCL requires tensors on a ROCm GPU device, got device: " + t.device().str());
-    if (!t.is_contiguous())
-        detail::fail<TensorError>("Tensor check failed: ", "t.is_contiguous()", nullptr, 0,
-                                  "MCCL v1 requires contiguous tensors. Call .contiguous() before passing to "
-                                  "collective.");
-    if (!detail::accepted_dtype(t.scalar_type()))
-        detail::fail<TensorError>("Tensor check failed: ", "accepted_dtype(t.scalar_type())", nullptr, 0,
-                                  std::string("MCCL supports float32/float16/bfloat16 (training), "
-                                              "int64/int32/bool/uint8 (metadata), and float64, got: ") +
-                                      at::toString(t.scalar_type()));
+    MCCL_CHECK_TENSOR(t.is_cuda(),
+                      "MCCL requires tensors on a ROCm GPU device, got device: " + t.device().str());
+    MCCL_CHECK_TENSOR(t.is_contiguous(),
+                      "MCCL v1 requires contiguous tensors. Call .contiguous() before passing to collective.");
+    const auto dt = t.scalar_type();
+    MCCL_CHECK_TENSOR(dt == at::kFloat || dt == at::kHalf || dt == at::kBFloat16 || dt == at::kLong ||
+                          dt == at::kInt || dt == at::kBool || dt == at::kByte || dt == at::kDouble,
+                      "MCCL supports float32/float16/bfloat16 (training), int64/int32/bool/uint8 "
+                      "(metadata), and float64, got: " + std::string(at::toString(dt)));
 }
 
 inline void check_same_shape_dtype(const at::Tensor& a, const at::Tensor& b) {
-    const bool same_shape = a.sizes() == b.sizes();
-    const bool same_dtype = a.scalar_type() == b.scalar_type();
-    if (!same_shape || !same_dtype)
-        detail::fail<TensorError>("Tensor check failed: ", same_shape ? "same dtype" : "same shape", nullptr, 0,
-                                  same_shape ? "Dtype mismatch in collective" : "Shape mismatch in collective");
+    MCCL_CHECK_TENSOR(a.sizes() == b.sizes(), "Shape mismatch in collective");
+    MCCL_CHECK_TENSOR(a.scalar_type() == b.scalar_type(), "Dtype mismatch in collective");
 }
 
-inline size_t tensor_nbytes(const at::Tensor& t) { return t.element_size() * static_cast<size_t>(t.numel()); }
+inline size_t tensor_nbytes(const at::Tensor& t) {
+    return static_cast<size_t>(t.numel()) * t.element_size();
+}
 
 struct HipBufferView {
     void* base;          // start of the storage

@@ -14,7 +14,12 @@ class TopKCompressor : public Compressor {
 public:
     explicit TopKCompressor(double k_ratio);
 
-    MCCL_COMPRESSOR_MEMBERS(, override)
+    size_t compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
+                    at::ScalarType dtype, uint64_t stable_id = 0) override;
+    void decompress(const void* src, size_t compressed_size, void* dst, size_t nbytes,
+                    at::ScalarType dtype) override;
+    size_t max_compressed_size(size_t nbytes) const override;
+    std::string name() const override { return "topk"; }
 
     void reset_error_feedback();
     void reset_error_feedback_for_tensor(uint64_t stable_id);

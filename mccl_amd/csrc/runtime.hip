@@ -21,9 +21,14 @@ Tuning g_tuning;
 thread_local int t_last_hip_error = 0;
 
 constexpr uint64_t kRing = 1024;
-hipEvent_t g_events[kRing];
-bool g_event_made[kRing];
-int g_event_device[kRing];
+constexpr int kMaxFenceDevices = 64;
+// One ring of events per device, created on first use and never destroyed (a
+// waiter may be polling an event outside the lock).  Slot s is owned by the
+// newest ticket t with t % kRing == s; g_slot_ticket names it, g_slot_device
+// the device whose ring holds its event.
+hipEvent_t* g_ring[kMaxFenceDevices];
+uint64_t g_slot_ticket[kRing];
+int g_slot_device[kRing];
 std::atomic<uint64_t> g_next_ticket{1};
 }  // namespace
 
@@ -70,11 +75,57 @@ const char* mccl_hip_strerror(int code) {
         case MCCL_HIP_ERR_RUNTIME: return "HIP runtime call failed";
         case MCCL_HIP_ERR_WORKSPACE: return "workspace too small";
         case MCCL_HIP_ERR_TIMEOUT: return "fence wait timed out";
+        case MCCL_HIP_ERR_POINTER: return "pointer is not GPU-accessible memory";
         default: return "unknown error";
     }
 }
 
 int mccl_hip_last_hip_error(void) { return t_last_hip_error; }
+
+int mccl_hip_pointer_check(const void* ptr, uint64_t nbytes, void** device_ptr) {
+    if (!ptr || !device_ptr) return MCCL_HIP_ERR_ARG;
+    int dev = -1;
+    MCCLHIP_TRY(hipGetDevice(&dev));
+    hipPointerAttribute_t attr;
+    hipError_t e = hipPointerGetAttributes(&attr, ptr);
+    if (e == hipErrorInvalidValue) {  // how older runtimes report memory they do not know
+        (void)hipGetLastError();
+        return MCCL_HIP_ERR_POINTER;
+    }
+    if (e != hipSuccess) {
+        record_hip_error(e);
+        (void)hipGetLastError();
+        return MCCL_HIP_ERR_RUNTIME;
+    }
+    void* dp = nullptr;
+    switch (attr.type) {
+        case hipMemoryTypeDevice: {
+            if (attr.device != dev) return MCCL_HIP_ERR_POINTER;
+            hipDeviceptr_t base = nullptr;
+            size_t size = 0;
+            e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return MCCL_HIP_ERR_POINTER;
+            }
+            const uintptr_t lo = (uintptr_t)base, p = (uintptr_t)ptr;
+            if (p < lo || nbytes > size || p - lo > size - nbytes) return MCCL_HIP_ERR_POINTER;
+            dp = const_cast<void*>(ptr);
+            break;
+        }
+        case hipMemoryTypeManaged:
+            dp = const_cast<void*>(ptr);
+            break;
+        case hipMemoryTypeHost:  // pinned: kernels reach it through its device-side alias
+            dp = attr.devicePointer;
+            if (!dp) return MCCL_HIP_ERR_POINTER;
+            break;
+        default:
+            return MCCL_HIP_ERR_POINTER;
+    }
+    *device_ptr = dp;
+    return MCCL_HIP_OK;
+}
 
 int mccl_hip_set_tuning(const char* key, int value) {
     if (!key) return MCCL_HIP_ERR_ARG;
@@ -109,36 +160,58 @@ int mccl_hip_fence_signal(void* stream, uint64_t* ticket) {
     std::lock_guard<std::mutex> lock(g_mu);
     int dev = -1;
     MCCLHIP_TRY(hipGetDevice(&dev));
-    uint64_t t = g_next_ticket.fetch_add(1);
-    uint64_t slot = t % kRing;
-    if (g_event_made[slot] && g_event_device[slot] != dev) {
-        MCCLHIP_TRY(hipEventDestroy(g_events[slot]));
-        g_event_made[slot] = false;
+    if (dev < 0 || dev >= kMaxFenceDevices) return MCCL_HIP_ERR_ARG;
+    if (!g_ring[dev]) {
+        hipEvent_t* ring = new hipEvent_t[kRing];
+        for (uint64_t i = 0; i < kRing; i++) {
+            hipError_t e = hipEventCreateWithFlags(&ring[i], hipEventDisableTiming);
+            if (e != hipSuccess) {
+                record_hip_error(e);
+                for (uint64_t j = 0; j < i; j++) (void)hipEventDestroy(ring[j]);
+                delete[] ring;
+                return MCCL_HIP_ERR_RUNTIME;
+            }
+        }
+        g_ring[dev] = ring;
     }
-    if (!g_event_made[slot]) {
-        MCCLHIP_TRY(hipEventCreateWithFlags(&g_events[slot], hipEventDisableTiming));
-        g_event_made[slot] = true;
-        g_event_device[slot] = dev;
+    const uint64_t t = g_next_ticket.load();
+    const uint64_t slot = t % kRing;
+    // The slot's previous owner (kRing tickets older) leaves the ring here.  "Left
+    // the ring" has to mean "complete" for every later wait on it, so its event is
+    // drained first; with per-step fences that are waited on promptly it already is.
+    if (g_slot_ticket[slot] != 0) {
+        hipEvent_t old = g_ring[g_slot_device[slot]][slot];
+        hipError_t e = hipEventQuery(old);
+        if (e == hipErrorNotReady) e = hipEventSynchronize(old);
+        if (e != hipSuccess) {
+            record_hip_error(e);
+            return MCCL_HIP_ERR_RUNTIME;
+        }
     }
-    MCCLHIP_TRY(hipEventRecord(g_events[slot], (hipStream_t)stream));
+    MCCLHIP_TRY(hipEventRecord(g_ring[dev][slot], (hipStream_t)stream));
+    g_slot_ticket[slot] = t;
+    g_slot_device[slot] = dev;
+    g_next_ticket.store(t + 1);
     *ticket = t;
     return MCCL_HIP_OK;
 }
 
-// 1 complete, 0 pending.  A ticket that has left the ring was signalled at
-// least kRing signals ago on an in-order stream of recorded events; its slot
-// now belongs to a newer ticket, whose completion is awaited instead (a
-// superset of what the caller asked for only when streams differ; tickets are
-// meant to be waited on promptly, as in the reference's per-step fences).
-static int fence_state(uint64_t ticket, hipEvent_t* ev) {
+// 1 complete, 0 pending (then *ev is the ticket's event), negative on error.  A
+// ticket whose slot has a newer owner was drained when that owner took the slot.
+static int fence_state_locked(uint64_t ticket, hipEvent_t* ev) {
     if (ticket == 0) return 1;
-    std::lock_guard<std::mutex> lock(g_mu);
-    uint64_t next = g_next_ticket.load();
-    if (ticket >= next) return MCCL_HIP_ERR_ARG;
-    uint64_t slot = ticket % kRing;
-    if (!g_event_made[slot]) return 1;
-    *ev = g_events[slot];
+    if (ticket >= g_next_ticket.load()) return MCCL_HIP_ERR_ARG;
+    const uint64_t slot = ticket % kRing;
+    if (g_slot_ticket[slot] != ticket) return 1;
+    *ev = g_ring[g_slot_device[slot]][slot];
     return 0;
+}
+// For host-side polling outside the lock: should the slot change owner while the
+// caller polls, the event then reports the newer ticket, recorded only after
+// this one had completed, so the caller still never returns early.
+static int fence_state(uint64_t ticket, hipEvent_t* ev) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    return fence_state_locked(ticket, ev);
 }
 
 int mccl_hip_fence_query(uint64_t ticket) {
@@ -173,8 +246,11 @@ int mccl_hip_fence_wait(uint64_t ticket, int timeout_ms) {
 }
 
 int mccl_hip_fence_block_stream(uint64_t ticket, void* stream) {
+    // under the lock: the wait must be enqueued on this ticket's record, not on a
+    // later record of the same event
+    std::lock_guard<std::mutex> lock(g_mu);
     hipEvent_t ev;
-    int st = fence_state(ticket, &ev);
+    int st = fence_state_locked(ticket, &ev);
     if (st < 0) return st;
     if (st == 1) return MCCL_HIP_OK;
     MCCLHIP_TRY(hipStreamWaitEvent((hipStream_t)stream, ev, 0));

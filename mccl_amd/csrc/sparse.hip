@@ -8,7 +8,7 @@
 // sparse accumulate: the reference decompresses every peer's payload into a
 // dense buffer and folds the dense buffers in ascending rank order
 // (csrc/backend/ProcessGroupMCCL.cpp:1692-1709,:2272-2296).  Here each block
-// owns one 4096-element tile of the output, keeps it in LDS starting at +0.0,
+// owns one 8192-element tile of the output, keeps it in LDS starting at +0.0,
 // and for rank 0, 1, ... adds that rank's pairs that fall inside the tile
 // (found by binary search in the sorted payload; indices are unique within a
 // rank, so a rank's adds never collide), then writes the tile once, scaled.

@@ -34,11 +34,20 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
-def _dev(t: torch.Tensor, what: str) -> None:
+def _dev(t: torch.Tensor, what: str, dtype: Optional[torch.dtype] = None, min_numel: int = 0) -> None:
+    """This layer is the only place buffer sizes are known: every tensor whose
+    pointer goes to the library is checked for device, layout, element type and
+    capacity here, so a short or host buffer raises instead of faulting the GPU."""
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{what} must be a tensor")
     if not t.is_cuda:
         raise ValueError(f"{what} must live on the GPU, got {t.device}")
     if not t.is_contiguous():
         raise ValueError(f"{what} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{what} must be {dtype}, got {t.dtype}")
+    if t.numel() < min_numel:
+        raise ValueError(f"{what} holds {t.numel()} elements, {min_numel} are needed")
 
 
 def fold2(dst: torch.Tensor, src: torch.Tensor, op: int = SUM) -> torch.Tensor:
@@ -79,6 +88,8 @@ def ring_fold(out: torch.Tensor, ins: Sequence[torch.Tensor], op: int = SUM,
         if t.numel() != out.numel() or t.dtype != out.dtype:
             raise ValueError("shape / dtype mismatch")
     n = out.numel()
+    if not ins:
+        raise ValueError("ring_fold needs at least one rank buffer")
     rc = _lib.load().mccl_hip_ring_fold(
         out.data_ptr(), _ptrs(ins), len(ins), n, bucket_elems or max(n, 1), schedule, dtype_code(out), op,
         0 if scale_by is None else 1, 0.0 if scale_by is None else scale_by, int(stepwise), _stream())
@@ -117,10 +128,14 @@ def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
     be = min(bucket_elems or n, n) if n else 1
     stride = wire_stride if wire_stride is not None else topk_wire_stride(be, ratio)
     nb = (n + be - 1) // be if n else 1
+    if residual.numel() != n:
+        raise ValueError(f"residual holds {residual.numel()} elements, the gradient {n}")
     if wire is None:
         wire = torch.empty(nb * stride, dtype=torch.uint8, device=grad.device)
     if workspace is None:
         workspace = topk_workspace(max(n, 1), be, ratio, grad.device)
+    _dev(wire, "wire", torch.uint8, nb * stride)
+    _dev(workspace, "workspace", torch.uint8)
     rc = _lib.load().mccl_hip_topk_compress(grad.data_ptr(), residual.data_ptr(), n, be, ratio,
                                            wire.data_ptr(), stride, workspace.data_ptr(),
                                            workspace.numel(), _stream())
@@ -139,13 +154,25 @@ def topk_path_report(workspace: torch.Tensor, n_total: int, bucket_elems: int, r
 
 def topk_decompress(wire: torch.Tensor, wire_bytes: int, count: int,
                     dense: Optional[torch.Tensor] = None, status: Optional[torch.Tensor] = None):
-    _dev(wire, "wire")
+    _dev(wire, "wire", torch.uint8, wire_bytes)
     if dense is None:
         dense = torch.empty(count, dtype=torch.float32, device=wire.device)
+    _dev(dense, "dense", torch.float32, count)
+    if status is not None:
+        _dev(status, "status", torch.int32, 1)
     rc = _lib.load().mccl_hip_topk_decompress(wire.data_ptr(), wire_bytes, dense.data_ptr(), count,
                                              None if status is None else status.data_ptr(), _stream())
     _lib.check(rc, "topk_decompress")
     return dense
+
+
+def _check_payload_sets(wires, n: int, bucket_elems: int, wire_stride: int, status) -> None:
+    be = max(1, min(bucket_elems, n))
+    nb = (n + be - 1) // be
+    for r, w in enumerate(wires):
+        _dev(w, f"wires[{r}]", torch.uint8, nb * wire_stride)
+    if status is not None:
+        _dev(status, "status", torch.int32, 1)
 
 
 def sparse_workspace(n_total: int, bucket_elems: int, ws: int, device) -> torch.Tensor:
@@ -159,11 +186,14 @@ def sparse_accumulate(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_str
                       bucket_elems: Optional[int] = None, scale_by: Optional[float] = None,
                       status: Optional[torch.Tensor] = None, workspace="auto") -> torch.Tensor:
     """workspace: "auto" allocates the scratch, None selects the scratch-free kernel."""
-    _dev(acc, "acc")
+    _dev(acc, "acc", torch.float32)
     n = acc.numel()
     be = bucket_elems or max(n, 1)
+    _check_payload_sets(wires, n, be, wire_stride, status)
     if isinstance(workspace, str):
         workspace = sparse_workspace(n, be, len(wires), acc.device)
+    if workspace is not None:
+        _dev(workspace, "workspace", torch.uint8)
     rc = _lib.load().mccl_hip_sparse_accumulate(
         acc.data_ptr(), n, be, _ptrs(wires), len(wires), wire_stride,
         0 if scale_by is None else 1, 0.0 if scale_by is None else scale_by,
@@ -175,18 +205,20 @@ def sparse_accumulate(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_str
 
 
 def cast_f32_to_f16(src: torch.Tensor, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
-    _dev(src, "src")
+    _dev(src, "src", torch.float32)
     if dst is None:
         dst = torch.empty(src.numel(), dtype=torch.float16, device=src.device)
+    _dev(dst, "dst", torch.float16, src.numel())
     _lib.check(_lib.load().mccl_hip_cast_f32_to_f16(src.data_ptr(), dst.data_ptr(), src.numel(), _stream()),
                "cast_f32_to_f16")
     return dst
 
 
 def cast_f16_to_f32(src: torch.Tensor, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
-    _dev(src, "src")
+    _dev(src, "src", torch.float16)
     if dst is None:
         dst = torch.empty(src.numel(), dtype=torch.float32, device=src.device)
+    _dev(dst, "dst", torch.float32, src.numel())
     _lib.check(_lib.load().mccl_hip_cast_f16_to_f32(src.data_ptr(), dst.data_ptr(), src.numel(), _stream()),
                "cast_f16_to_f32")
     return dst

@@ -55,3 +55,26 @@ def test_argument_errors_need_no_gpu():
     assert lib.mccl_hip_fold2(None, None, 4, 6, 5, None) == -1         # BAND unsupported
     assert lib.mccl_hip_fold2(None, None, 4, 6, 0, None) == -6         # null pointer
     assert lib.mccl_hip_topk_decompress(ctypes.c_void_p(4096), 7, ctypes.c_void_p(4096), 8, None, None) == -4
+
+
+def test_tensor_layer_rejects_host_buffers_before_any_call():
+    # the ctypes layer knows the buffer sizes; host tensors and short buffers raise ValueError there
+    import torch
+    from mccl_amd import hip_ops as ops
+    a = torch.zeros(8)
+    for call in (lambda: ops.fold2(a, a.clone()), lambda: ops.scale(a, 0.5), lambda: ops.fold2_scale(a, a.clone(), 0.5),
+                 lambda: ops.ring_fold(a, [a.clone(), a.clone()]),
+                 lambda: ops.topk_compress(a, a.clone(), 0.5),
+                 lambda: ops.topk_decompress(torch.zeros(12, dtype=torch.uint8), 12, 8),
+                 lambda: ops.sparse_accumulate(a, [torch.zeros(12, dtype=torch.uint8)], 12),
+                 lambda: ops.cast_f32_to_f16(a), lambda: ops.cast_f16_to_f32(a.half())):
+        with pytest.raises(ValueError, match="must live on the GPU"):
+            call()
+
+
+def test_pointer_check_needs_arguments():
+    from mccl_amd import _lib
+    lib = _lib.load()
+    out = ctypes.c_void_p(0)
+    assert lib.mccl_hip_pointer_check(None, 16, ctypes.byref(out)) == -6
+    assert lib.mccl_hip_strerror(-10) == b"pointer is not GPU-accessible memory"

@@ -268,3 +268,30 @@ def test_sparse_accumulate_flags_bad_payloads(ops):
     bad = good.copy(); bad[4:20] = np.array([9_999, 0x3F800000, 5, 0x40000000], "<u4").view(np.uint8)
     ops.sparse_accumulate(acc, [torch.from_numpy(bad).to(DEV)], stride, status=status)
     assert int(status) == oracle.ERR_INDEX
+
+
+def test_tensor_layer_checks_secondary_buffers(ops):
+    # a short or mistyped buffer raises in the ctypes layer, before the library sees a pointer
+    g = torch.zeros(1000, device=DEV)
+    with pytest.raises(ValueError, match="residual holds"):
+        ops.topk_compress(g, torch.zeros(999, device=DEV), 0.1)
+    with pytest.raises(ValueError, match="wire holds"):
+        ops.topk_compress(g, g.clone(), 0.1, wire=torch.empty(16, dtype=torch.uint8, device=DEV))
+    with pytest.raises(ValueError, match="workspace must live on the GPU"):
+        ops.topk_compress(g, g.clone(), 0.1, workspace=torch.empty(1 << 20, dtype=torch.uint8))
+    wire, stride = ops.topk_compress(g, g.clone(), 0.1)
+    with pytest.raises(ValueError, match="wire holds"):
+        ops.topk_decompress(wire, wire.numel() + 8, 1000)
+    with pytest.raises(ValueError, match="dense holds"):
+        ops.topk_decompress(wire, 4 + 8 * 100, 1000, dense=torch.empty(999, device=DEV))
+    with pytest.raises(ValueError, match="status must be torch.int32"):
+        ops.topk_decompress(wire, 4 + 8 * 100, 1000, status=torch.zeros(1, device=DEV))
+    acc = torch.empty(1000, device=DEV)
+    with pytest.raises(ValueError, match=r"wires\[1\] holds"):
+        ops.sparse_accumulate(acc, [wire, wire[:100]], stride)
+    with pytest.raises(ValueError, match=r"wires\[0\] must live on the GPU"):
+        ops.sparse_accumulate(acc, [wire.cpu()], stride)
+    with pytest.raises(ValueError, match="dst holds"):
+        ops.cast_f32_to_f16(g, torch.empty(10, dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError, match="dst must be torch.float32"):
+        ops.cast_f16_to_f32(g.half(), torch.empty(1000, dtype=torch.float16, device=DEV))
