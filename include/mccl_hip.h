@@ -201,6 +201,21 @@ int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_ele
  * every block, which costs about 3x the time on MI355X. */
 uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, int ws);
 
+/* mccl_hip_sparse_accumulate for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments, meaning and
+ * results as mccl_hip_sparse_accumulate with a workspace, but the tile-bounds
+ * table lives in a MCCL_HIP_SPARSE_STATIC_BYTES array inside the library's
+ * device image (one copy per GPU, held until the process ends), and the call
+ * itself allocates nothing.  Shapes whose table
+ * (mccl_hip_sparse_accumulate_workspace_bytes) exceeds that size are refused
+ * with MCCL_HIP_ERR_WORKSPACE.  All calls on one GPU share the array: calls
+ * that may overlap on one GPU (different streams without ordering) race. */
+#define MCCL_HIP_SPARSE_STATIC_BYTES (2u << 20)
+int mccl_hip_sparse_accumulate_static(float* acc, uint64_t n_total, uint64_t bucket_elems,
+                                      const void* const* host_wires, int ws, uint64_t wire_stride,
+                                      int apply_scale, float scale, int* status, void* stream);
+
 /* ---- fp16 transport casts ------------------------------------------------ */
 
 /* FP16Compressor's casts (csrc/compression/FP16Compression.cpp:16-112):

@@ -31,6 +31,7 @@ SIGNATURES = {
     "mccl_hip_topk_decompress": (_i32, [_vp, _u64, _vp, _u64, _vp, _vp]),
     "mccl_hip_sparse_accumulate": (_i32, [_vp, _u64, _u64, C.POINTER(_vp), _i32, _u64, _i32, _f32, _vp, _vp, _u64, _vp]),
     "mccl_hip_sparse_accumulate_workspace_bytes": (_u64, [_u64, _u64, _i32]),
+    "mccl_hip_sparse_accumulate_static": (_i32, [_vp, _u64, _u64, C.POINTER(_vp), _i32, _u64, _i32, _f32, _vp, _vp]),
     "mccl_hip_cast_f32_to_f16": (_i32, [_vp, _vp, _u64, _vp]),
     "mccl_hip_cast_f16_to_f32": (_i32, [_vp, _vp, _u64, _vp]),
     "mccl_hip_fence_signal": (_i32, [_vp, C.POINTER(_u64)]),

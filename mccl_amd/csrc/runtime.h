@@ -36,6 +36,10 @@ void record_hip_error(hipError_t e);
         }                                            \
     } while (0)
 
+// sparse.hip: resolves the current device's copy of the static scratch array of
+// mccl_hip_sparse_accumulate_static (once per device, from mccl_hip_init).
+int sparse_static_setup(int device);
+
 // Call after every kernel launch: launch-time errors surface here.
 inline int launch_status() {
     hipError_t e = hipGetLastError();

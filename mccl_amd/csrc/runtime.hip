@@ -57,6 +57,8 @@ int mccl_hip_init(void) {
         record_hip_error(hipErrorNoBinaryForGpu);
         return MCCL_HIP_ERR_RUNTIME;
     }
+    int rc = sparse_static_setup(dev);
+    if (rc) return rc;
     g_info.device = dev;
     g_info.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     g_info.ok = true;

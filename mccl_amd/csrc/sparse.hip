@@ -58,6 +58,16 @@ struct WirePtrs {
     const uint8_t* w[MCCL_HIP_MAX_WORLD];
 };
 
+// Scratch of mccl_hip_sparse_accumulate_static: the tile-bounds table lives in
+// this file-scope device array instead of a caller workspace, so the call
+// allocates nothing.  Every GPU holds its own copy at its own address; host
+// code only ever uses the address hipGetSymbolAddress returned for the device
+// (g_static_ptr), never the array's name.
+constexpr uint64_t kStaticWords = MCCL_HIP_SPARSE_STATIC_BYTES / 4;
+static __device__ __align__(256) uint32_t scratch[kStaticWords];
+constexpr int kMaxDevices = 64;
+uint32_t* g_static_ptr[kMaxDevices];
+
 // First pair position in [0, k) whose index is >= target (k if none).
 __device__ __forceinline__ uint32_t lower_bound_idx(const uint32_t* pairs, uint32_t k, uint32_t target) {
     uint32_t lo = 0, hi = k;
@@ -287,7 +297,58 @@ __global__ __launch_bounds__(kAccThreads) void k_sparse_accumulate_b(float* acc,
     }
 }
 
+// Validates the arguments and enqueues the kernels; `workspace` (may be null:
+// scratch-free kernel) is known to be large enough.
+int accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems, const void* const* host_wires, int ws,
+               uint64_t wire_stride, int apply_scale, float scale, int* status, void* workspace,
+               void* stream) {
+    if (!acc || !host_wires || ws < 1 || ws > MCCL_HIP_MAX_WORLD) return MCCL_HIP_ERR_ARG;
+    if (n_total == 0 || n_total > MCCL_HIP_MAX_ELEMS || bucket_elems == 0) return MCCL_HIP_ERR_ARG;
+    if (wire_stride < 4 || (wire_stride & 3)) return MCCL_HIP_ERR_ARG;
+    if (bucket_elems > n_total) bucket_elems = n_total;
+    if (bucket_elems > 0xFFFFFFFFull) return MCCL_HIP_ERR_ARG;
+    const uint64_t nb = (n_total + bucket_elems - 1) / bucket_elems;
+    if (nb * (uint64_t)ws > 65535) return MCCL_HIP_ERR_ARG;
+    WirePtrs wp;
+    for (int r = 0; r < MCCL_HIP_MAX_WORLD; r++) wp.w[r] = nullptr;
+    for (int r = 0; r < ws; r++) {
+        if (!host_wires[r] || ((uintptr_t)host_wires[r] & 3)) return MCCL_HIP_ERR_ARG;
+        wp.w[r] = (const uint8_t*)host_wires[r];
+    }
+    int rc = mccl_hip_init();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const uint32_t tiles = (uint32_t)((bucket_elems + kAccTile - 1) / kAccTile);
+    if (!workspace) {
+        // no scratch: every block finds its ranges by binary search
+        k_sparse_accumulate<<<dim3(tiles, (uint32_t)nb), kBlock, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
+                                                                           wire_stride, apply_scale, scale, status);
+        return launch_status();
+    }
+    uint32_t* start = (uint32_t*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
+    const uint64_t kmax = (wire_stride - 4) / 8;
+    const uint32_t bx = clamp_u32((kmax + kBlock * 8 - 1) / (kBlock * 8), 1, 0x7FFFFFFF);
+    k_sparse_bounds<<<dim3(bx, (uint32_t)(nb * ws)), kBlock, 0, st>>>(wp, ws, wire_stride, n_total, bucket_elems,
+                                                                        tiles, start, status);
+    k_sparse_accumulate_b<<<dim3(tiles, (uint32_t)nb), kAccThreads, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
+                                                                         wire_stride, tiles, start, apply_scale,
+                                                                         scale, status);
+    return launch_status();
+}
+
 }  // namespace
+
+// Called by mccl_hip_init with `device` current, once per device: looks up the
+// address of that device's copy of the static scratch array.
+int sparse_static_setup(int device) {
+    if (device < 0 || device >= kMaxDevices) return MCCL_HIP_OK;  // the static entry point reports it
+    if (g_static_ptr[device]) return MCCL_HIP_OK;
+    uint32_t* p = nullptr;
+    MCCLHIP_TRY(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+    g_static_ptr[device] = p;
+    return MCCL_HIP_OK;
+}
+
 }  // namespace mcclhip
 
 using namespace mcclhip;
@@ -325,40 +386,24 @@ int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_ele
                                const void* const* host_wires, int ws, uint64_t wire_stride,
                                int apply_scale, float scale, int* status, void* workspace,
                                uint64_t workspace_bytes, void* stream) {
-    if (!acc || !host_wires || ws < 1 || ws > MCCL_HIP_MAX_WORLD) return MCCL_HIP_ERR_ARG;
-    if (n_total == 0 || n_total > MCCL_HIP_MAX_ELEMS || bucket_elems == 0) return MCCL_HIP_ERR_ARG;
-    if (wire_stride < 4 || (wire_stride & 3)) return MCCL_HIP_ERR_ARG;
-    if (bucket_elems > n_total) bucket_elems = n_total;
-    if (bucket_elems > 0xFFFFFFFFull) return MCCL_HIP_ERR_ARG;
-    const uint64_t nb = (n_total + bucket_elems - 1) / bucket_elems;
-    if (nb * (uint64_t)ws > 65535) return MCCL_HIP_ERR_ARG;
-    WirePtrs wp;
-    for (int r = 0; r < MCCL_HIP_MAX_WORLD; r++) wp.w[r] = nullptr;
-    for (int r = 0; r < ws; r++) {
-        if (!host_wires[r] || ((uintptr_t)host_wires[r] & 3)) return MCCL_HIP_ERR_ARG;
-        wp.w[r] = (const uint8_t*)host_wires[r];
-    }
     if (workspace && workspace_bytes < mccl_hip_sparse_accumulate_workspace_bytes(n_total, bucket_elems, ws))
         return MCCL_HIP_ERR_WORKSPACE;
-    int rc = mccl_hip_init();
+    return accumulate(acc, n_total, bucket_elems, host_wires, ws, wire_stride, apply_scale, scale, status,
+                      workspace, stream);
+}
+
+int mccl_hip_sparse_accumulate_static(float* acc, uint64_t n_total, uint64_t bucket_elems,
+                                      const void* const* host_wires, int ws, uint64_t wire_stride,
+                                      int apply_scale, float scale, int* status, void* stream) {
+    const uint64_t need = mccl_hip_sparse_accumulate_workspace_bytes(n_total, bucket_elems, ws);
+    if (need == 0) return MCCL_HIP_ERR_ARG;
+    if (need > MCCL_HIP_SPARSE_STATIC_BYTES) return MCCL_HIP_ERR_WORKSPACE;
+    int rc = mccl_hip_init();  // resolves this device's copy of the scratch array on first use
     if (rc) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    const uint32_t tiles = (uint32_t)((bucket_elems + kAccTile - 1) / kAccTile);
-    if (!workspace) {
-        // no scratch: every block finds its ranges by binary search
-        k_sparse_accumulate<<<dim3(tiles, (uint32_t)nb), kBlock, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
-                                                                           wire_stride, apply_scale, scale, status);
-        return launch_status();
-    }
-    uint32_t* start = (uint32_t*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
-    const uint64_t kmax = (wire_stride - 4) / 8;
-    const uint32_t bx = clamp_u32((kmax + kBlock * 8 - 1) / (kBlock * 8), 1, 0x7FFFFFFF);
-    k_sparse_bounds<<<dim3(bx, (uint32_t)(nb * ws)), kBlock, 0, st>>>(wp, ws, wire_stride, n_total, bucket_elems,
-                                                                        tiles, start, status);
-    k_sparse_accumulate_b<<<dim3(tiles, (uint32_t)nb), kAccThreads, 0, st>>>(acc, n_total, bucket_elems, wp, ws,
-                                                                         wire_stride, tiles, start, apply_scale,
-                                                                         scale, status);
-    return launch_status();
+    const int dev = device_info().device;
+    if (dev < 0 || dev >= kMaxDevices || !g_static_ptr[dev]) return MCCL_HIP_ERR_RUNTIME;
+    return accumulate(acc, n_total, bucket_elems, host_wires, ws, wire_stride, apply_scale, scale, status,
+                      g_static_ptr[dev], stream);
 }
 
 }  // extern "C"

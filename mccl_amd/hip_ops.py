@@ -204,6 +204,21 @@ def sparse_accumulate(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_str
     return acc
 
 
+def sparse_accumulate_static(acc: torch.Tensor, wires: Sequence[torch.Tensor], wire_stride: int,
+                             bucket_elems: Optional[int] = None, scale_by: Optional[float] = None,
+                             status: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """sparse_accumulate on the library's static scratch: the call allocates nothing."""
+    _dev(acc, "acc", torch.float32)
+    n = acc.numel()
+    _check_payload_sets(wires, n, bucket_elems or max(n, 1), wire_stride, status)
+    rc = _lib.load().mccl_hip_sparse_accumulate_static(
+        acc.data_ptr(), n, bucket_elems or max(n, 1), _ptrs(wires), len(wires), wire_stride,
+        0 if scale_by is None else 1, 0.0 if scale_by is None else scale_by,
+        None if status is None else status.data_ptr(), _stream())
+    _lib.check(rc, "sparse_accumulate_static")
+    return acc
+
+
 def cast_f32_to_f16(src: torch.Tensor, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
     _dev(src, "src", torch.float32)
     if dst is None:

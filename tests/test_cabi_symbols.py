@@ -67,6 +67,7 @@ def test_tensor_layer_rejects_host_buffers_before_any_call():
                  lambda: ops.topk_compress(a, a.clone(), 0.5),
                  lambda: ops.topk_decompress(torch.zeros(12, dtype=torch.uint8), 12, 8),
                  lambda: ops.sparse_accumulate(a, [torch.zeros(12, dtype=torch.uint8)], 12),
+                 lambda: ops.sparse_accumulate_static(a, [torch.zeros(12, dtype=torch.uint8)], 12),
                  lambda: ops.cast_f32_to_f16(a), lambda: ops.cast_f16_to_f32(a.half())):
         with pytest.raises(ValueError, match="must live on the GPU"):
             call()

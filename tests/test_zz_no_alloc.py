@@ -1,0 +1,63 @@
+"""mccl_hip_sparse_accumulate_static (the entry point that allocates nothing: its
+tile-bounds table is a static device array) against mccl_hip_sparse_accumulate
+with a caller workspace, bit for bit, through the C ABI: two calls in a row,
+the second on a smaller input, so stale contents of the shared array from the
+first call are in place when the second runs."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests._gpu_util import DEV, to_np, bits, student_t
+
+pytestmark = pytest.mark.gpu
+F32 = oracle.F32
+
+
+def payloads(rng, ws, n, be, ratio):
+    nb = (n + be - 1) // be
+    stride = 4 + 8 * (int(be * ratio) + 1)
+    shared = rng.random(n) < 0.004
+    out = []
+    for _ in range(ws):
+        g = student_t(rng, n, ties=0.0)
+        g[shared] *= 50.0
+        buf = np.zeros(nb * stride, np.uint8)
+        for b in range(nb):
+            s, e = b * be, min(n, (b + 1) * be)
+            w, rc = oracle.topk_compress(g[s:e].copy(), np.zeros(e - s, np.float32), ratio)
+            buf[b * stride: b * stride + rc] = w
+        out.append(torch.from_numpy(buf).to(DEV))
+    return out, stride
+
+
+def test_static_scratch_entry_point_matches_workspace_entry_point():
+    from mccl_amd import hip_ops as ops
+    from mccl_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(2025)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    # first a large call (many tiles, 8 ranks), then a smaller one with other bucket geometry
+    for ws, n, be, ratio in ((8, 3_000_017, 655_360, 0.01), (3, 200_003, 65_536, 0.02)):
+        wires, stride = payloads(rng, ws, n, be, ratio)
+        want = torch.full((n,), 3.0, device=DEV)
+        ops.sparse_accumulate(want, wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status,
+                              workspace="auto")
+        got = torch.full((n,), 5.0, device=DEV)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        ops.sparse_accumulate_static(got, wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == before
+        assert int(status) == 0
+        assert np.array_equal(bits(to_np(got, F32)), bits(to_np(want, F32))), (ws, n, be)
+    # a shape whose bounds table does not fit the static array is refused, nothing is launched
+    ws, n, be = 64, 200_000_000, 100_000_000
+    need = lib.mccl_hip_sparse_accumulate_workspace_bytes(n, be, ws)
+    assert need > 2 << 20
+    ptrs = (C.c_void_p * ws)(*[wires[0].data_ptr()] * ws)
+    rc = lib.mccl_hip_sparse_accumulate_static(got.data_ptr(), n, be, ptrs, ws, 4 + 8 * 1_000_001, 0, 0.0,
+                                               None, None)
+    assert rc == -8
