@@ -85,7 +85,10 @@ enum {
     S_ISTAR = 8,          // fast path: ties are taken while index <= this
     S_EXACT_HIST = 9,     // 1 when hist round 0 holds the full histogram
     S_N2 = 10,            // fast path: entries in list2
-    S_THAT = 13           // fast path: predicted threshold key; pass A stores 0 for keys >= this
+    S_THAT = 13,          // fast path: predicted threshold key; pass A stores 0 for keys >= this
+    S_BAR1 = 14,          // fused tail: blocks of the bucket that have flushed their histogram
+    S_BAR2 = 15,          // fused tail: blocks that have published their certain picks and list2 share
+    S_TIMEOUT = 16        // fused tail: a block gave up waiting at a barrier (result invalid)
 };
 
 struct Geometry {
@@ -112,6 +115,7 @@ struct Workspace {
     uint32_t* reg_off;      // [nbuckets][regions] picks in all regions before it
     uint32_t* list;         // [nbuckets][regions][kRegSlots][2]  (index, bits), index order
     uint32_t* list2;        // [nbuckets][lcap2][2] candidates of the threshold bin (index, key)
+    uint32_t* blk_above;    // [nbuckets][kNSub] fused tail: picks above the threshold bin per block
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -957,7 +961,8 @@ __global__ __launch_bounds__(kBlock) void k_topk_select1(const float* residual, 
 // Whole exact selection of one bucket by one block: the fallback for buckets
 // whose candidate lists turned out incomplete.  Slow (one block streams the
 // bucket five times) but costs no extra launch: select2 calls it in place.
-// lh: kBins0 words, scratch: kSelThreads / kWave + 2 words of LDS.
+// lh: kBins0 words, scratch: THREADS / kWave + 2 words of LDS.
+template <int THREADS>
 __device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uint8_t* wire, uint64_t wire_stride,
                              uint32_t* lh, uint32_t* scratch) {
     const uint64_t bn = bucket_count(g, b);
@@ -967,16 +972,16 @@ __device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uin
         const int bins = round == 0 ? kBins0 : kBinsR;
         const int shift = round == 0 ? 20 : (round == 1 ? 10 : 0);
         const int hi_shift = round == 0 ? 31 : shift + 10;
-        for (int i = threadIdx.x; i < kBins0; i += kSelThreads) lh[i] = 0;
+        for (int i = threadIdx.x; i < kBins0; i += THREADS) lh[i] = 0;
         __syncthreads();
-        for (uint64_t i = threadIdx.x; i < bn; i += kSelThreads) {
+        for (uint64_t i = threadIdx.x; i < bn; i += THREADS) {
             const uint32_t key = key_of(rp[i]);
             if ((key >> hi_shift) == (prefix >> hi_shift)) atomicAdd(&lh[(key >> shift) & (bins - 1)], 1u);
         }
         __syncthreads();
         uint32_t left, bin;
-        if (round == 0) bin = pick_bin<kBins0, kSelThreads>(lh, remaining, 0, &left, scratch);
-        else bin = pick_bin<kBinsR, kSelThreads>(lh, remaining, 0, &left, scratch);
+        if (round == 0) bin = pick_bin<kBins0, THREADS>(lh, remaining, 0, &left, scratch);
+        else bin = pick_bin<kBinsR, THREADS>(lh, remaining, 0, &left, scratch);
         prefix |= bin << shift;
         remaining = left;
     }
@@ -984,14 +989,14 @@ __device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uin
     uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
     if (threadIdx.x == 0) out[0] = bucket_k(g, b);
     uint32_t gt_run = 0, eq_run = 0;
-    for (uint64_t base = 0; base < bn; base += kSelThreads) {
+    for (uint64_t base = 0; base < bn; base += THREADS) {
         const uint64_t i = base + threadIdx.x;
         const uint32_t bitsv = i < bn ? f2u(rp[i]) : 0u;
         const uint32_t key = bitsv & 0x7FFFFFFFu;
         const bool is_gt = i < bn && key > T;
         const bool is_eq = i < bn && key == T;
         uint32_t total;
-        const uint32_t ex = block_exclusive_scan_n<kSelThreads>((is_gt ? 1u : 0u) + (is_eq ? 0x10000u : 0u), scratch,
+        const uint32_t ex = block_exclusive_scan_n<THREADS>((is_gt ? 1u : 0u) + (is_eq ? 0x10000u : 0u), scratch,
                                                                 &total);
         const uint32_t gt_b = gt_run + (ex & 0xFFFFu), eq_b = eq_run + (ex >> 16);
         if (is_gt || (is_eq && eq_b < need)) {
@@ -1008,13 +1013,14 @@ __device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uin
 // Puts back the values pass A replaced by 0.0f (listed candidates with key >=
 // the predicted threshold) so that the exact fallback sees the plain sums.
 // Called by all threads of a select2 block.
+template <int THREADS>
 __device__ void restore_prezeroed(float* residual, const Geometry& g, const Workspace& w, uint32_t b) {
     const uint32_t that_key = w.state[(uint64_t)b * kStateWords + S_THAT];
     const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
     const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
     const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
     float* rp = residual + (uint64_t)b * g.bucket_elems;
-    for (uint32_t slot = threadIdx.x; slot < nreg * kRegSlots; slot += kSelThreads) {
+    for (uint32_t slot = threadIdx.x; slot < nreg * kRegSlots; slot += THREADS) {
         const uint32_t cnt = rc[slot / kRegSlots];
         if (cnt == kDense || (slot % kRegSlots) >= cnt) continue;
         const uint32_t idx = lb[2 * (uint64_t)slot], bitsv = lb[2 * (uint64_t)slot + 1];
@@ -1041,8 +1047,8 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     if (jstar >= (uint32_t)(kWinBins - 1) || count2 > g.lcap2) {
         // threshold outside the window, or more keys in its bin than list2 holds (rare):
         // this block runs the whole exact selection of the bucket; S_OK stays 0, so emit skips it
-        restore_prezeroed(residual, g, w, b);
-        bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
+        restore_prezeroed<kSelThreads>(residual, g, w, b);
+        bucket_exact<kSelThreads>(residual, g, b, wire, wire_stride, lh, scratch);
         return;
     }
 
@@ -1149,8 +1155,8 @@ __global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, G
     }
     if (total != bucket_k(g, b)) {  // uniform; cannot happen with consistent lists
         __syncthreads();
-        restore_prezeroed(residual, g, w, b);
-        bucket_exact(residual, g, b, wire, wire_stride, lh, scratch);
+        restore_prezeroed<kSelThreads>(residual, g, w, b);
+        bucket_exact<kSelThreads>(residual, g, b, wire, wire_stride, lh, scratch);
     }
 }
 
@@ -1229,6 +1235,447 @@ __global__ __launch_bounds__(kBlock) void k_topk_emit_fast(float* residual, Geom
     }
 }
 
+// ================================ fused tail ======================================
+// Everything after the streaming pass in one launch: window histogram, threshold
+// bin, exact threshold, tie-break, payload offsets and the payload itself.  The
+// kNSub blocks that work on one bucket meet at two barriers (the histogram is
+// complete; the threshold bin's candidates and the blocks' certain-pick counts
+// are published); nothing else crosses blocks.  Each wavefront owns a contiguous
+// run of regions and keeps their slots in registers across the phases, so the
+// candidate lists are read from memory once.
+//
+// Barrier: a per-bucket arrival counter in the state words (zero at kernel
+// start).  A block's 64 partners are the blocks next to it in dispatch order, so
+// they are resident or about to be; the wait is bounded all the same: a block
+// that waits longer than `limit_ticks` of the 100 MHz wall clock records
+// S_TIMEOUT and leaves, and the call's result for that bucket is then invalid
+// (mccl_hip_topk_path_report returns an error).
+
+constexpr int kTailRegs = 14;  // regions per wavefront whose slots stay in registers
+
+__device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// All threads of the block call it.  Returns false when the wait timed out.
+// Everything blocks hand to each other goes through agent-scope stores, atomics
+// and loads (they bypass the per-XCD L2 copies), so the barrier needs no cache
+// write-back or invalidate: each wavefront only waits until its own stores and
+// atomics have been acknowledged before the block's arrival is counted.  (Whole-
+// cache fences here, repeated by a thousand polling blocks, made the kernel ten
+// times slower.)
+__device__ __forceinline__ bool bucket_barrier(uint32_t* counter, uint32_t parties, uint32_t* flag /* LDS */,
+                                               uint64_t limit_ticks) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint64_t t0 = 0;
+        uint32_t ok = 1, polls = 0;
+        while (ld_agent(counter) < parties) {
+            __builtin_amdgcn_s_sleep(8);
+            if ((++polls & 63u) == 0) {  // look at the clock now and then
+                const uint64_t now = (uint64_t)wall_clock64();
+                if (t0 == 0) t0 = now;
+                else if (now - t0 > limit_ticks) {
+                    ok = 0;
+                    break;
+                }
+            }
+        }
+        *flag = ok;
+    }
+    __syncthreads();
+    return *flag != 0;
+}
+
+// Dense regions (more candidates than slots) are rare.  Every sweep of the tail
+// kernel handles them in a compact loop of its own after the unrolled sweep over
+// the wavefront's register-held regions, so the common path stays small.
+// Calls f(index, bits, in_range) for every element of dense region r, 64 elements
+// per step, every lane of the wavefront taking part in every step; the loads of
+// 16 steps are in flight together and parked in LDS, so the code stays a loop.
+template <class F>
+__device__ __forceinline__ void dense_walk(const float* rp, uint64_t bn, uint32_t r, uint32_t* buf /* 1024 words of LDS per wavefront */,
+                                           F&& f) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint64_t e0 = (uint64_t)r * kRegion;
+    const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
+    constexpr int B = 16;
+#pragma unroll 1
+    for (uint64_t base = e0; base < e1; base += (uint64_t)B * kWave) {
+        uint32_t v[B];
+#pragma unroll
+        for (int j = 0; j < B; j++) {
+            const uint64_t i = base + (uint64_t)j * kWave + lane;
+            v[j] = i < e1 ? f2u(rp[i]) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < B; j++) buf[j * kWave + lane] = v[j];  // a lane reads back only what it wrote
+#pragma unroll 1
+        for (int j = 0; j < B && base + (uint64_t)j * kWave < e1; j++) {  // wave-uniform trip count
+            const uint64_t i = base + (uint64_t)j * kWave + lane;
+            f((uint32_t)i, buf[j * kWave + lane], i < e1);
+        }
+    }
+}
+
+// The need-th smallest index among list2's entries with key == T (ties at the
+// threshold go to the lower index): radix select over the index, 11 + 11 + 10 bits.
+// Called by all threads of the block.
+__device__ __forceinline__ uint32_t resolve_ties(const uint32_t* l2, uint32_t count2, uint32_t T, uint32_t need,
+                                              uint32_t* lh /* kBins0 words */, uint32_t* scratch) {
+    uint32_t iwant = need, iprefix = 0;
+    const int shifts[3] = {21, 10, 0};
+    const int widths[3] = {11, 11, 10};
+    for (int r = 0; r < 3; r++) {
+        const int bins = 1 << widths[r];
+        for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
+        __syncthreads();
+        const int hs = shifts[r] + widths[r];
+        for (uint32_t i = threadIdx.x; i < count2; i += kBlock) {
+            const uint32_t idx = ld_agent(&l2[2 * (uint64_t)i]), key = ld_agent(&l2[2 * (uint64_t)i + 1]);
+            const bool match = hs >= 32 ? true : ((idx >> hs) == (iprefix >> hs));
+            // bins stored reversed, so that pick_bin's top-down scan runs over ascending indices
+            if (key == T && match) atomicAdd(&lh[(bins - 1) - ((idx >> shifts[r]) & (bins - 1))], 1u);
+        }
+        __syncthreads();
+        uint32_t left;
+        // a 1024-bin round leaves the upper half of the 2048 bins empty: one scan serves both widths
+        const uint32_t rb = pick_bin<kBins0, kBlock>(lh, iwant, 0, &left, scratch);
+        iprefix |= ((uint32_t)(bins - 1) - (rb - (uint32_t)(kBins0 - bins))) << shifts[r];
+        iwant = left;
+    }
+    return iprefix;
+}
+
+// The bucket goes to the exact selection (run by one block; S_OK stays 0).
+__device__ __forceinline__ void tail_fallback(float* residual, const Geometry& g, const Workspace& w, uint32_t b,
+                                           uint8_t* wire, uint64_t wire_stride, uint32_t* lh, uint32_t* scratch) {
+    restore_prezeroed<kBlock>(residual, g, w, b);
+    bucket_exact<kBlock>(residual, g, b, wire, wire_stride, lh, scratch);
+}
+
+__global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geometry g, Workspace w, uint8_t* wire,
+                                                         uint64_t wire_stride, uint64_t limit_ticks) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ uint32_t lh[kBins0];
+    __shared__ uint32_t scratch[NW + 2];
+    __shared__ uint32_t sh_a[NW], sh_b[NW], sh_x[2];
+    __shared__ uint32_t rcnt[NW][kTailRegs];  // phase 4: picks per register-held region
+    __shared__ uint32_t dbuf[NW][16 * kWave];  // dense_walk's staging area, one per wavefront
+    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT], that_key = st[S_THAT];
+    const uint32_t k = bucket_k(g, b);
+    const uint64_t bn = bucket_count(g, b);
+    uint32_t r0, r1;
+    block_regions(g, b, s, &r0, &r1);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const uint64_t below = (1ull << lane) - 1ull;
+    // this wavefront's regions: a contiguous quarter of the block's
+    const uint32_t pw = (r1 - r0 + NW - 1) / NW;
+    const uint32_t wr0 = r0 + wave * pw < r1 ? r0 + wave * pw : r1;
+    const uint32_t wr1 = wr0 + pw < r1 ? wr0 + pw : r1;
+    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
+    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    uint32_t* hw = w.hist_w + (uint64_t)b * kWinBins;
+    uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
+    uint32_t* above_of = w.blk_above + (uint64_t)b * kNSub;
+    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
+
+    // ---- slots of the first kTailRegs regions into registers, every load issued at once
+    uint32_t ccnt[kTailRegs], cidx[kTailRegs], cbits[kTailRegs];
+#pragma unroll
+    for (int q = 0; q < kTailRegs; q++) {
+        const uint32_t r = wr0 + q < wr1 ? wr0 + q : (wr1 > wr0 ? wr1 - 1 : 0);  // stays inside the bucket's lists
+        ccnt[q] = rc[r];
+        const u2a e = *(const u2a*)(lb + 2 * ((uint64_t)r * kRegSlots + lane));  // slots past the count: ignored below
+        cidx[q] = e[0];
+        cbits[q] = e[1];
+    }
+    bool any_dense = false;  // wave-uniform: one of the register-held regions is dense
+#pragma unroll
+    for (int q = 0; q < kTailRegs; q++) any_dense |= wr0 + q < wr1 && ccnt[q] == kDense;
+
+    // A sweep = nd(q, r, cnt, idx, bits) for every ordinary region (q < kTailRegs: register-held,
+    // else ~0u), dn(q, r) for every dense one.  Order: register-held ordinary regions first, then
+    // the dense ones and those past the register window, in index order.
+    const bool more = any_dense || wr1 > wr0 + kTailRegs;  // wave-uniform
+    auto sweep = [&](auto&& nd, auto&& dn) {
+#pragma unroll
+        for (int q = 0; q < kTailRegs; q++)
+            if (wr0 + q < wr1 && ccnt[q] != kDense) nd((uint32_t)q, wr0 + q, ccnt[q], cidx[q], cbits[q]);
+        if (more) {
+#pragma unroll 1
+            for (uint32_t r = wr0; r < wr1; r++) {
+                const uint32_t q = r - wr0 < (uint32_t)kTailRegs ? r - wr0 : ~0u;
+                const uint32_t cnt = rc[r];
+                if (cnt == kDense) {
+                    dn(q, r);
+                } else if (q == ~0u) {
+                    const u2a e = *(const u2a*)(lb + 2 * ((uint64_t)r * kRegSlots + lane));
+                    nd(q, r, cnt, e[0], e[1]);
+                }
+            }
+        }
+    };
+    // Reasons to hand the bucket to the exact selection are collected in `failed`
+    // (block-uniform, and the same in every block of the bucket); the one call sits
+    // at the end of the kernel.
+    bool failed = false;
+
+    // ---- phase 1: window histogram -------------------------------------------------
+    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
+    __syncthreads();
+    sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t, uint32_t bitsv) {
+              if ((uint32_t)lane < cnt) atomicAdd(&lh[window_bin(bitsv & 0x7FFFFFFFu, lo, hi, shift)], 1u);
+          },
+          [&](uint32_t, uint32_t r) {
+              dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
+                  const uint32_t key = v & 0x7FFFFFFFu;
+                  if (in && key >= lo) atomicAdd(&lh[window_bin(key, lo, hi, shift)], 1u);
+              });
+          });
+    __syncthreads();
+    for (int i = threadIdx.x; i < kWinBins; i += kBlock) {
+        const uint32_t c = lh[i];
+        if (c) __hip_atomic_fetch_add(&hw[i], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!bucket_barrier(st + S_BAR1, kNSub, &sh_x[0], limit_ticks)) {
+        if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
+        return;
+    }
+
+    do {
+    // ---- phase 2: threshold bin; certain picks per block; the bin's candidates to list2
+    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = ld_agent(&hw[i]);
+    __syncthreads();
+    uint32_t need;
+    const uint32_t jstar = pick_bin<kWinBins, kBlock>(lh, k, 0, &need, scratch);
+    if (jstar >= (uint32_t)(kWinBins - 1)) {  // fewer than k candidates, or the threshold lies above the window
+        failed = true;
+        break;
+    }
+    uint32_t w_above = 0, w_hits = 0;
+    sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t, uint32_t bitsv) {
+              const bool valid = (uint32_t)lane < cnt;
+              const uint32_t bin = valid ? window_bin(bitsv & 0x7FFFFFFFu, lo, hi, shift) : 0u;
+              w_above += (uint32_t)__popcll(__ballot(valid && bin > jstar));
+              w_hits += (uint32_t)__popcll(__ballot(valid && bin == jstar));
+          },
+          [&](uint32_t, uint32_t r) {
+              dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
+                  const uint32_t key = v & 0x7FFFFFFFu;
+                  const bool cand = in && key >= lo;
+                  const uint32_t bin = cand ? window_bin(key, lo, hi, shift) : 0u;
+                  w_above += (uint32_t)__popcll(__ballot(cand && bin > jstar));
+                  w_hits += (uint32_t)__popcll(__ballot(cand && bin == jstar));
+              });
+          });
+    if (lane == 0) { sh_a[wave] = w_above; sh_b[wave] = w_hits; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t ta = 0, th = 0;
+#pragma unroll
+        for (int i = 0; i < NW; i++) { ta += sh_a[i]; th += sh_b[i]; }
+        st_agent(&above_of[s], ta);
+        sh_x[1] = th ? __hip_atomic_fetch_add(st + S_N2, th, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    }
+    __syncthreads();
+    if (w_hits) {  // wave-uniform; list2's order does not matter
+        uint32_t pos = sh_x[1];
+        for (int i = 0; i < wave; i++) pos += sh_b[i];
+        auto put = [&](bool hit, uint32_t idx, uint32_t key) {
+            const uint64_t m = __ballot(hit);
+            if (hit) {
+                const uint32_t p = pos + (uint32_t)__popcll(m & below);
+                if (p < g.lcap2) {
+                    st_agent(&l2[2 * (uint64_t)p], idx);
+                    st_agent(&l2[2 * (uint64_t)p + 1], key);
+                }
+            }
+            pos += (uint32_t)__popcll(m);
+        };
+        sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t idx, uint32_t bitsv) {
+                  const uint32_t key = bitsv & 0x7FFFFFFFu;
+                  put((uint32_t)lane < cnt && window_bin(key, lo, hi, shift) == jstar, idx, key);
+              },
+              [&](uint32_t, uint32_t r) {
+                  dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
+                      const uint32_t key = v & 0x7FFFFFFFu;
+                      put(in && key >= lo && window_bin(key, lo, hi, shift) == jstar, i, key);
+                  });
+              });
+    }
+    if (!bucket_barrier(st + S_BAR2, kNSub, &sh_x[0], limit_ticks)) {
+        if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
+        return;
+    }
+
+    // ---- phase 3: exact threshold from list2 (every block, redundantly) -----------------
+    const uint32_t count2 = ld_agent(st + S_N2);
+    if (count2 > g.lcap2) {  // more keys in the threshold bin than list2 holds (heavy ties)
+        failed = true;
+        break;
+    }
+    constexpr int kL2Regs = 4;  // list2 entries per thread kept in registers (1024 per block)
+    uint32_t eidx[kL2Regs], ekey[kL2Regs];
+#pragma unroll
+    for (int j = 0; j < kL2Regs; j++) {
+        const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
+        eidx[j] = i < count2 ? ld_agent(&l2[2 * (uint64_t)i]) : 0u;
+        ekey[j] = i < count2 ? ld_agent(&l2[2 * (uint64_t)i + 1]) : 0u;
+    }
+    auto for_list2 = [&](auto&& body) {
+#pragma unroll
+        for (int j = 0; j < kL2Regs; j++)
+            if ((uint32_t)j * kBlock + threadIdx.x < count2) body(eidx[j], ekey[j]);
+#pragma unroll 1
+        for (uint32_t i = kL2Regs * kBlock + threadIdx.x; i < count2; i += kBlock)
+            body(ld_agent(&l2[2 * (uint64_t)i]), ld_agent(&l2[2 * (uint64_t)i + 1]));
+    };
+    const uint32_t bin_lo = lo + (jstar << shift);  // smallest key of the threshold bin
+    uint32_t vprefix = 0, want = need;              // key - bin_lo: up to 30 bits, selected as 10 + 10 + 10
+    // a window bin spans 2^shift keys: rounds whose digits lie wholly above that are skipped
+    const int first_round = shift <= 10 ? 2 : (shift <= 20 ? 1 : 0);
+#pragma unroll 1
+    for (int r = first_round; r < 3; r++) {
+        const int sh = 20 - 10 * r;
+        const int hs = sh + 10;
+        for (int i = threadIdx.x; i < kBinsR; i += kBlock) lh[i] = 0;
+        __syncthreads();
+        for_list2([&](uint32_t, uint32_t key) {
+            const uint32_t v = key - bin_lo;
+            if ((v >> hs) == (vprefix >> hs)) atomicAdd(&lh[(v >> sh) & (kBinsR - 1)], 1u);
+        });
+        __syncthreads();
+        uint32_t left;
+        const uint32_t bin = pick_bin<kBinsR, kBlock>(lh, want, 0, &left, scratch);
+        vprefix |= bin << sh;
+        want = left;
+    }
+    const uint32_t T = bin_lo + vprefix;
+    const uint32_t need2 = want;
+    const uint32_t ties = lh[vprefix & (kBinsR - 1)];
+    __syncthreads();
+    // when only some keys equal to T are taken, they are the need2 lowest indices
+    const uint32_t istar = ties != need2 ? resolve_ties(l2, count2, T, need2, lh, scratch) : 0xFFFFFFFFu;
+    auto is_pick = [&](bool valid, uint32_t key, uint32_t idx) {
+        return valid && (key > T || (key == T && idx <= istar));
+    };
+    // picks before this block's first element: the earlier blocks' certain picks and the
+    // threshold bin's picks at lower indices
+    uint32_t mine_before = 0, mine_all = 0;
+    const uint64_t first_elem = (uint64_t)r0 * kRegion;
+    for_list2([&](uint32_t idx, uint32_t key) {
+        if (is_pick(true, key, idx)) {
+            mine_all++;
+            mine_before += (uint64_t)idx < first_elem ? 1u : 0u;
+        }
+    });
+    uint32_t l2_before, l2_total, above_before, above_total;
+    block_exclusive_scan(mine_before, scratch, &l2_before);
+    block_exclusive_scan(mine_all, scratch, &l2_total);
+    {
+        const uint32_t v = threadIdx.x < (uint32_t)kNSub ? ld_agent(&above_of[threadIdx.x]) : 0u;
+        block_exclusive_scan(threadIdx.x < s ? v : 0u, scratch, &above_before);
+        block_exclusive_scan(v, scratch, &above_total);
+    }
+    if (above_total + l2_total != k) {  // cannot happen with consistent lists
+        failed = true;
+        break;
+    }
+
+    // ---- phase 4: payload, in index order -----------------------------------------------
+    // picks per region first: the register-held regions' into rcnt, the others' into a total
+    uint32_t w_total = 0;
+    sweep([&](uint32_t q, uint32_t, uint32_t cnt, uint32_t idx, uint32_t bitsv) {
+              const uint32_t c = (uint32_t)__popcll(__ballot(is_pick((uint32_t)lane < cnt, bitsv & 0x7FFFFFFFu, idx)));
+              if (q != ~0u) rcnt[wave][q] = c;
+              w_total += c;
+          },
+          [&](uint32_t q, uint32_t r) {
+              uint32_t c = 0;
+              dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
+                  c += (uint32_t)__popcll(__ballot(is_pick(in, v & 0x7FFFFFFFu, i)));
+              });
+              if (q != ~0u) rcnt[wave][q] = c;
+              w_total += c;
+          });
+    if (lane == 0) sh_a[wave] = w_total;
+    __syncthreads();
+    uint32_t wave_off = above_before + l2_before;
+    for (int i = 0; i < wave; i++) wave_off += sh_a[i];
+    auto emit_dense = [&](uint32_t r, uint32_t pos) {
+        dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
+            const bool pick = is_pick(in, v & 0x7FFFFFFFu, i);
+            const uint64_t m = __ballot(pick);
+            if (pick) {
+                const uint32_t p = pos + (uint32_t)__popcll(m & below);
+                out[1 + 2 * (uint64_t)p] = i;
+                out[2 + 2 * (uint64_t)p] = v;
+                rp[i] = 0.0f;
+            }
+            pos += (uint32_t)__popcll(m);
+        });
+        return pos;
+    };
+    auto emit_region = [&](uint32_t cnt, uint32_t idx, uint32_t bitsv, uint32_t pos) {
+        const bool valid = (uint32_t)lane < cnt;
+        const uint32_t key = bitsv & 0x7FFFFFFFu;
+        const bool pick = is_pick(valid, key, idx);
+        const uint64_t m = __ballot(pick);
+        if (pick) {
+            const u2a e = {idx, bitsv};
+            *(u2a4*)(out + 1 + 2 * (uint64_t)(pos + (uint32_t)__popcll(m & below))) = e;
+        }
+        // pass A stored 0.0f for key >= predicted threshold; repair where the prediction was wrong
+        if (valid && pick != (key >= that_key)) rp[idx] = pick ? 0.0f : u2f(bitsv);
+        return pos + (uint32_t)__popcll(m);
+    };
+    {
+        uint32_t pos = wave_off;
+#pragma unroll
+        for (int q = 0; q < kTailRegs; q++) {
+            if (wr0 + q < wr1) {
+                if (ccnt[q] != kDense) pos = emit_region(ccnt[q], cidx[q], cbits[q], pos);
+                else pos += rcnt[wave][q];  // written out by the loop below
+            }
+        }
+    }
+    if (more) {
+        uint32_t pos = wave_off;
+#pragma unroll 1
+        for (uint32_t r = wr0; r < wr1; r++) {
+            const uint32_t cnt = rc[r];
+            if (cnt == kDense) {
+                pos = emit_dense(r, pos);
+            } else if (r - wr0 < (uint32_t)kTailRegs) {
+                pos += rcnt[wave][r - wr0];
+            } else {
+                const u2a e = *(const u2a*)(lb + 2 * ((uint64_t)r * kRegSlots + lane));
+                pos = emit_region(cnt, e[0], e[1], pos);
+            }
+        }
+    }
+    if (s == 0 && threadIdx.x == 0) {
+        out[0] = k;
+        st[S_T] = T;
+        st[S_NEED] = need2;
+        st[S_ISTAR] = istar;
+        st[S_OK] = 1u;
+    }
+    } while (false);
+    // the exact selection for a bucket the window could not finish: one block runs it, S_OK stays 0
+    if (failed && s == 0) tail_fallback(residual, g, w, b, wire, wire_stride, lh, scratch);
+}
+
 // ================================ host side =======================================
 
 uint64_t align4(uint64_t words) { return (words + 3) & ~uint64_t(3); }
@@ -1241,7 +1688,8 @@ uint64_t zeroed_words(const Geometry& g) {
 uint64_t workspace_words(const Geometry& g) {
     return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) +
            3 * align4((uint64_t)g.nbuckets * g.regions) +
-           align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2) + align4((uint64_t)g.nbuckets * g.lcap2 * 2);
+           align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2) + align4((uint64_t)g.nbuckets * g.lcap2 * 2) +
+           align4((uint64_t)g.nbuckets * kNSub);
 }
 
 Workspace carve(void* base, const Geometry& g) {
@@ -1256,7 +1704,8 @@ Workspace carve(void* base, const Geometry& g) {
     w.reg_pick = p;    p += align4((uint64_t)g.nbuckets * g.regions);
     w.reg_off = p;     p += align4((uint64_t)g.nbuckets * g.regions);
     w.list = p;        p += align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2);
-    w.list2 = p;
+    w.list2 = p;       p += align4((uint64_t)g.nbuckets * g.lcap2 * 2);
+    w.blk_above = p;
     return w;
 }
 
@@ -1337,10 +1786,18 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
         k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(grad, residual, g, w);
         const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
-        k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
-        k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
-        k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
-        k_topk_emit_fast<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
+        if (tuning().topk_tail == 0) {
+            // 100 MHz ticks a block may wait at a barrier before it gives up
+            const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
+            k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride,
+                                                                    limit);
+        } else {
+            k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
+            k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
+            k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
+            k_topk_emit_fast<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire,
+                                                                         wire_stride);
+        }
     } else {
         const uint64_t zw = zeroed_words(g);
         k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);
@@ -1366,7 +1823,10 @@ int mccl_hip_topk_path_report(const void* workspace, uint64_t n_total, uint64_t 
     MCCLHIP_TRY(hipMemcpyAsync(st.data(), w.state, st.size() * 4, hipMemcpyDeviceToHost, (hipStream_t)stream));
     MCCLHIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     uint32_t ok = 0;
-    for (uint32_t b = 0; b < g.nbuckets; b++) ok += st[(size_t)b * kStateWords + S_OK] ? 1u : 0u;
+    for (uint32_t b = 0; b < g.nbuckets; b++) {
+        if (st[(size_t)b * kStateWords + S_TIMEOUT]) return MCCL_HIP_ERR_TIMEOUT;  // the payload is invalid
+        ok += st[(size_t)b * kStateWords + S_OK] ? 1u : 0u;
+    }
     *host_single_pass_buckets = ok;
     *host_buckets = g.nbuckets;
     return MCCL_HIP_OK;

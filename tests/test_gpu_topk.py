@@ -32,7 +32,8 @@ def oracle_buckets(g, r, ratio, be):
     return wires, res
 
 
-PATHS = {"exact": 1, "single-pass": 2}  # both must give the oracle's bytes on every input
+# (topk_path, topk_tail): all must give the oracle's bytes on every input
+PATHS = {"exact": (1, 0), "single-pass": (2, 0), "single-pass, four tail kernels": (2, 1)}
 
 
 def check_compress(ops, g, r, ratio, be=None, pad=0):
@@ -40,10 +41,14 @@ def check_compress(ops, g, r, ratio, be=None, pad=0):
     be = be or n
     want_wires, want_res = oracle_buckets(g, r, ratio, be)
     try:
-        for name, path in PATHS.items():
+        for name, (path, tail) in PATHS.items():
             ops.set_tuning("topk_path", path)
+            ops.set_tuning("topk_tail", tail)
             dg = to_dev(g, F32, pad); dr = to_dev(r, F32, pad)
-            wire, stride = ops.topk_compress(dg, dr, ratio, bucket_elems=be)
+            ws = ops.topk_workspace(n, min(be, n), ratio, DEV)
+            wire, stride = ops.topk_compress(dg, dr, ratio, bucket_elems=be, workspace=ws)
+            if path == 2:
+                ops.topk_path_report(ws, n, min(be, n), ratio)   # raises if a bucket barrier timed out
             torch.cuda.synchronize()
             got_res = to_np(dr, F32)
             assert np.array_equal(bits(got_res), bits(want_res)), name
@@ -54,6 +59,7 @@ def check_compress(ops, g, r, ratio, be=None, pad=0):
                 assert got.tobytes() == ww.tobytes(), f"{name}: bucket {b}"
     finally:
         ops.set_tuning("topk_path", 0)
+        ops.set_tuning("topk_tail", 0)
     return wire, stride, want_wires
 
 
