@@ -163,6 +163,15 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
                            uint64_t wire_stride, void* workspace, uint64_t workspace_bytes,
                            void* stream);
 
+/* The workspace carries state from one call to the next: after a call it holds,
+ * per bucket, the exact threshold just found, and the next call with the same
+ * workspace and shape starts from it instead of sampling the gradient again (a
+ * wrong prediction costs time, never correctness: the bucket is then selected
+ * exactly).  Use one workspace per gradient tensor.  Call this before the memory
+ * is freed or reused for something else, or to make the next call sample afresh.
+ * No counterpart in the reference. */
+int mccl_hip_topk_workspace_forget(void* workspace);
+
 /* Diagnostics, no counterpart in the reference: after a compress call on
  * `stream` has been enqueued with this workspace and shape, waits for the
  * stream and reports how many buckets were finished by the single-pass path
@@ -251,7 +260,7 @@ int mccl_hip_fence_block_stream(uint64_t ticket, void* stream);
 int mccl_hip_sync(void* stream);
 
 /* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
-/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path" */
+/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_warm", "topk_barrier_ms" */
 int mccl_hip_set_tuning(const char* key, int value);
 int mccl_hip_get_tuning(const char* key);
 

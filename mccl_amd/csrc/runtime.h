@@ -22,7 +22,7 @@ struct Tuning {
     int fold_blocks_per_cu = 256;  // grid cap of the streaming kernels, in blocks per CU
     int nontemporal = 1;         // 1: streaming loads/stores carry the `nt` hint (+8..12 % on MI355X)
     int topk_path = 0;           // 0 auto, 1 multi-pass exact path only, 2 single-pass path at any size
-    int topk_tail = 0;           // single-pass path: 0 fused tail kernel, 1 four separate tail kernels
+    int topk_warm = 0;           // single-pass path: 1 start from the previous call's threshold instead of a sample (stationary gradients only)
     int topk_barrier_ms = 2000;  // fused tail: longest wait of a block at a bucket barrier
 };
 Tuning& tuning();

@@ -49,6 +49,8 @@
 #include "common.hip.h"
 #include "runtime.h"
 
+#include <mutex>
+#include <unordered_map>
 #include <vector>
 
 namespace mcclhip {
@@ -68,7 +70,6 @@ static_assert(kATile == kRegion * (kBlock / kWave), "one region per wavefront");
 static_assert(kRegSlots == kWave, "a wavefront reads a region's slots in one go");
 constexpr uint32_t kDense = 0xFFFFFFFFu;  // region count: more candidates than slots, read the residual range itself
 constexpr int kNSub = 64;      // fast path: blocks per bucket in the kernels that walk the regions
-constexpr int kSelThreads = 1024;
 constexpr int kSampleThreads = 1024;  // sample kernel (256 threads measured slower: 21 vs 15.5 us)
 constexpr uint64_t kFastMinBucket = 1u << 18;
 constexpr int kSample = 12288;  // fast path: sampled elements per bucket (12 per select thread)
@@ -88,8 +89,48 @@ enum {
     S_THAT = 13,          // fast path: predicted threshold key; pass A stores 0 for keys >= this
     S_BAR1 = 14,          // fused tail: blocks of the bucket that have flushed their histogram
     S_BAR2 = 15,          // fused tail: blocks that have published their certain picks and list2 share
-    S_TIMEOUT = 16        // fused tail: a block gave up waiting at a barrier (result invalid)
+    S_TIMEOUT = 16,       // fused tail: a block gave up waiting at a barrier (result invalid)
+    // The window words (S_LO_KEY, S_HI_KEY, S_SHIFT, S_THAT) and the next three survive from
+    // call to call: after every call they hold the window predicted for the next one.
+    S_DLO = 17,           // predicted threshold minus lower window end, in key units (from the last sample)
+    S_DHI = 18,           // upper window end minus predicted threshold
+    S_WARM = 19,          // 1 once a call has left a prediction behind
+    S_BARF = 20           // 20..23: barriers of the in-kernel exact selection
 };
+
+// The shared description of a bucket's window, and the rule every kernel applies to
+// whatever the state words hold (they may be stale or arbitrary when a caller hands
+// in a workspace with foreign contents): elements are only ever stored as zero when
+// they are also listed, i.e. the predicted threshold is never below the window.
+struct Window {
+    uint32_t lo, hi, shift, that;
+    bool sound;  // bins fit the histogram; otherwise the bucket takes the exact selection
+};
+__device__ __forceinline__ Window load_window(const uint32_t* st) {
+    Window wn;
+    wn.lo = st[S_LO_KEY];
+    wn.hi = st[S_HI_KEY];
+    wn.shift = st[S_SHIFT];
+    wn.that = st[S_THAT] < wn.lo ? wn.lo : st[S_THAT];
+    wn.sound = wn.shift < 32u && wn.hi >= wn.lo && ((wn.hi - wn.lo) >> (wn.shift & 31u)) < (uint32_t)(kWinBins - 1);
+    wn.shift &= 31u;
+    return wn;
+}
+// Block (0, b) of a call's last kernel: the window for the next call, centred on this call's
+// exact threshold with the widths the last sample found.
+__device__ __forceinline__ void predict_next_window(uint32_t* st, uint32_t T) {
+    const uint32_t dlo = st[S_DLO], dhi = st[S_DHI];
+    const uint32_t lo = T > dlo ? T - dlo : 0u;
+    uint32_t hi = dhi < 0x7FFFFFFFu - T ? T + dhi : 0x7FFFFFFFu;
+    if (hi < lo) hi = lo;
+    uint32_t shift = 0;
+    while (((hi - lo) >> shift) >= (uint32_t)(kWinBins - 1)) shift++;
+    st[S_LO_KEY] = lo;
+    st[S_HI_KEY] = hi;
+    st[S_SHIFT] = shift;
+    st[S_THAT] = T < lo ? lo : T;
+    st[S_WARM] = 1u;
+}
 
 struct Geometry {
     uint64_t n_total;
@@ -111,11 +152,10 @@ struct Workspace {
     uint32_t* tile_gt;      // [nbuckets][tiles]
     uint32_t* tile_eq;      // [nbuckets][tiles]
     uint32_t* reg_cnt;      // [nbuckets][regions] candidates in the region's slots, or kDense
-    uint32_t* reg_pick;     // [nbuckets][regions] picks in the region
-    uint32_t* reg_off;      // [nbuckets][regions] picks in all regions before it
     uint32_t* list;         // [nbuckets][regions][kRegSlots][2]  (index, bits), index order
     uint32_t* list2;        // [nbuckets][lcap2][2] candidates of the threshold bin (index, key)
     uint32_t* blk_above;    // [nbuckets][kNSub] fused tail: picks above the threshold bin per block
+    uint32_t* blk_eq;       // [nbuckets][kNSub] in-kernel exact selection: keys equal to the threshold per block
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -503,9 +543,6 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __r
     __shared__ uint32_t lh[3][kBinsR];
     __shared__ uint32_t scratch[3 * (kSampleThreads / kWave + 2)];
     const uint32_t b = blockIdx.x;
-    // this bucket's accumulators for the kernels that follow start at zero
-    for (int i = threadIdx.x; i < kWinBins; i += kSampleThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
-    if (threadIdx.x < kStateWords) w.state[(uint64_t)b * kStateWords + threadIdx.x] = 0;
     const uint64_t bn = bucket_count(g, b);
     const float* gp = grad + (uint64_t)b * g.bucket_elems;
     const float* rp = residual + (uint64_t)b * g.bucket_elems;
@@ -591,7 +628,12 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __r
         st[S_SHIFT] = shift;
         // never below lo: every pre-zeroed element must be a listed candidate
         uint32_t that = active[2] ? prefix[2] : 0x7FFFFFFFu;
-        st[S_THAT] = that < lo ? lo : that;
+        if (that < lo) that = lo;
+        st[S_THAT] = that;
+        // widths for the predictions that follow this call
+        st[S_DLO] = that - lo;
+        st[S_DHI] = hi > that ? hi - that : 0u;
+        st[S_WARM] = 1u;
     }
 }
 
@@ -602,90 +644,6 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __r
 // reg_cnt.  A region with more candidates than slots is marked kDense: readers
 // then take every element of the region's residual range as a candidate.  No
 // atomics and no shared capacity are involved, so nothing can overflow.
-
-// One chunk of a block's slot range: kChunk slots per thread, all loads issued
-// before the first use.  A wavefront's 64 lanes cover exactly one region per j.
-constexpr int kChunk = 8;
-struct SlotChunk {
-    uint32_t idx[kChunk], bits[kChunk], region[kChunk];
-    bool valid[kChunk];   // the slot holds a candidate
-    uint32_t dense_mask;  // bit j: the region of slot j is dense
-};
-__device__ __forceinline__ SlotChunk load_slots(const uint32_t* reg_cnt_b, const uint32_t* list_b, uint32_t slot0,
-                                                uint32_t slot_end) {
-    SlotChunk c;
-    uint32_t cnt[kChunk];
-    c.dense_mask = 0;
-#pragma unroll
-    for (int j = 0; j < kChunk; j++) {
-        const uint32_t slot = slot0 + (uint32_t)j * kBlock + threadIdx.x;
-        c.region[j] = slot / kRegSlots;
-        cnt[j] = slot < slot_end ? reg_cnt_b[c.region[j]] : 0u;
-    }
-#pragma unroll
-    for (int j = 0; j < kChunk; j++) {
-        const uint32_t slot = slot0 + (uint32_t)j * kBlock + threadIdx.x;
-        c.dense_mask |= (cnt[j] == kDense ? 1u : 0u) << j;
-        c.valid[j] = cnt[j] != kDense && (slot % kRegSlots) < cnt[j];
-        u2a e = {0u, 0u};
-        if (c.valid[j]) e = *(const u2a*)(list_b + 2 * (uint64_t)slot);
-        c.idx[j] = e[0];
-        c.bits[j] = e[1];
-    }
-    return c;
-}
-
-// Dense regions met by a block are noted in LDS while it walks its slots (one
-// lane per region notes it), so the rare dense work is a loop over that short
-// list.  dl[0] counts, dl[1..kDenseList] hold region numbers; when more dense
-// regions turn up than fit, the caller walks all its regions instead.
-constexpr uint32_t kDenseList = 62;
-__device__ __forceinline__ void note_dense(const SlotChunk& c, uint32_t* dl) {
-    if (c.dense_mask && (threadIdx.x & (kWave - 1)) == 0) {
-#pragma unroll
-        for (int j = 0; j < kChunk; j++) {
-            if ((c.dense_mask >> j) & 1u) {
-                const uint32_t p = atomicAdd(&dl[0], 1u);
-                if (p < kDenseList) dl[1 + p] = c.region[j];
-            }
-        }
-    }
-}
-// The i-th dense region a wavefront should handle next, or ~0u when there is none.
-// `r` walks [r0, r1) when the list overflowed.
-__device__ __forceinline__ uint32_t next_dense(const uint32_t* dl, const uint32_t* rc, uint32_t* cursor, uint32_t r0,
-                                               uint32_t r1) {
-    const uint32_t n = dl[0];
-    const uint32_t step = kBlock / kWave;
-    if (n <= kDenseList) {
-        const uint32_t i = *cursor;
-        if (i >= n) return ~0u;
-        *cursor = i + step;
-        return dl[1 + i];
-    }
-    for (uint32_t r = r0 + *cursor; r < r1; r += step) {
-        if (rc[r] == kDense) {
-            *cursor = r - r0 + step;
-            return r;
-        }
-    }
-    return ~0u;
-}
-
-// Copies the bit patterns of a dense region's elements [e0, e1) into this
-// wavefront's kRegion words of LDS, every load issued before the first store, so
-// that the loops over a dense region are not a chain of dependent HBM reads.
-__device__ __forceinline__ void stage_region(const float* rp, uint64_t e0, uint64_t e1, uint32_t* buf) {
-    const int lane = threadIdx.x & (kWave - 1);
-    uint32_t v[kRegion / kWave];
-#pragma unroll
-    for (int it = 0; it < kRegion / kWave; it++) {
-        const uint64_t i = e0 + (uint64_t)it * kWave + lane;
-        v[it] = i < e1 ? f2u(rp[i]) : 0u;
-    }
-#pragma unroll
-    for (int it = 0; it < kRegion / kWave; it++) buf[it * kWave + lane] = v[it];
-}
 
 // The regions [r0, r1) of bucket b that block s of kNSub works on.
 __device__ __forceinline__ void block_regions(const Geometry& g, uint32_t b, uint32_t s, uint32_t* r0, uint32_t* r1) {
@@ -714,6 +672,17 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const uint64_t w0 = (uint64_t)t * kATile + (uint64_t)wave * kRegion;  // first element of this wave's region
+    if (t == 0) {
+        // the words the selection kernel accumulates into start every call at zero
+        static_assert(kWinBins == kBlock, "one histogram bin per thread");
+        w.hist_w[(uint64_t)b * kWinBins + threadIdx.x] = 0;
+        if (threadIdx.x == 0) {
+            uint32_t* st = w.state + (uint64_t)b * kStateWords;
+            st[S_BAR1] = 0; st[S_BAR2] = 0; st[S_N2] = 0; st[S_OK] = 0; st[S_TIMEOUT] = 0;
+            st[S_BARF] = 0; st[S_BARF + 1] = 0; st[S_BARF + 2] = 0; st[S_BARF + 3] = 0;
+        }
+        for (int i = threadIdx.x; i < kHistWords; i += kBlock) w.hist[(uint64_t)b * kHistWords + i] = 0;
+    }
     if (w0 >= bn) return;  // whole wavefront; the kernel has no barriers
     const float* gp = grad + (uint64_t)b * g.bucket_elems + w0;
     float* rp = residual + (uint64_t)b * g.bucket_elems + w0;
@@ -735,8 +704,8 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         }
     };
     issue(0);
-    const uint32_t lo_key = w.state[(uint64_t)b * kStateWords + S_LO_KEY];
-    const uint32_t that_key = w.state[(uint64_t)b * kStateWords + S_THAT];
+    const Window wn = load_window(w.state + (uint64_t)b * kStateWords);
+    const uint32_t lo_key = wn.lo, that_key = wn.that;
     const uint64_t below = (1ull << lane) - 1ull;
     uint32_t staged = 0;  // wave-uniform
     bool dense = false;   // wave-uniform: more candidates than slots
@@ -822,419 +791,6 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
     if (lane == 0) w.reg_cnt[(uint64_t)b * g.regions + region] = dense ? kDense : staged;
 }
 
-// Window histogram of a bucket's candidates: kNSub blocks per bucket, counts in
-// LDS, one flush per block.
-__global__ __launch_bounds__(kBlock) void k_topk_window_hist(const float* residual, Geometry g, Workspace w) {
-    __shared__ uint32_t lh[kWinBins];
-    __shared__ uint32_t dl[kDenseList + 2];
-    __shared__ uint32_t dreg[kBlock / kWave][kRegion];
-    const uint32_t b = blockIdx.y;
-    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
-    uint32_t r0, r1;
-    block_regions(g, b, blockIdx.x, &r0, &r1);
-    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
-    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
-    if (threadIdx.x == 0) dl[0] = 0;
-    __syncthreads();
-    for (uint32_t s0 = r0 * kRegSlots; s0 < r1 * kRegSlots; s0 += kChunk * kBlock) {
-        const SlotChunk c = load_slots(rc, lb, s0, r1 * kRegSlots);
-        note_dense(c, dl);
-#pragma unroll
-        for (int j = 0; j < kChunk; j++)
-            if (c.valid[j]) atomicAdd(&lh[window_bin(c.bits[j] & 0x7FFFFFFFu, lo, hi, shift)], 1u);
-    }
-    __syncthreads();
-    if (dl[0]) {  // rare: some region of this block's range is dense
-        const uint64_t bn = bucket_count(g, b);
-        const float* rp = residual + (uint64_t)b * g.bucket_elems;
-        uint32_t cursor = threadIdx.x / kWave;
-        for (uint32_t r; (r = next_dense(dl, rc, &cursor, r0, r1)) != ~0u;) {
-            const uint64_t e0 = (uint64_t)r * kRegion;
-            const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
-            uint32_t* buf = dreg[threadIdx.x / kWave];
-            stage_region(rp, e0, e1, buf);
-            for (uint32_t i = threadIdx.x & (kWave - 1); i < (uint32_t)(e1 - e0); i += kWave) {
-                const uint32_t key = buf[i] & 0x7FFFFFFFu;
-                if (key >= lo) atomicAdd(&lh[window_bin(key, lo, hi, shift)], 1u);
-            }
-        }
-    }
-    __syncthreads();
-    flush_hist<kBlock>(lh, w.hist_w + (uint64_t)b * kWinBins, kWinBins);
-}
-
-// select, step 1: finds the window bin that holds the k-th largest key (every
-// block gets the same answer), counts per region the candidates in higher bins
-// (picks for certain) and copies the threshold bin's candidates to list2 (order
-// irrelevant): the rest of the selection only touches those.
-__global__ __launch_bounds__(kBlock) void k_topk_select1(const float* residual, Geometry g, Workspace w) {
-    __shared__ uint32_t scratch[kBlock / kWave + 2];
-    __shared__ uint32_t gbase;
-    __shared__ uint32_t dl[kDenseList + 2];
-    __shared__ uint32_t dreg[kBlock / kWave][kRegion];
-    const uint32_t b = blockIdx.y;
-    uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT];
-    if (threadIdx.x == 0) dl[0] = 0;  // pick_bin's barriers publish it
-    uint32_t need;
-    const uint32_t jstar = pick_bin<kWinBins, kBlock>(w.hist_w + (uint64_t)b * kWinBins, bucket_k(g, b), 0, &need, scratch);
-    if (blockIdx.x == 0 && threadIdx.x == 0) { st[S_P0] = jstar; st[S_R0] = need; }
-    // fewer than k candidates, or the threshold lies above the window: fallback
-    if (jstar >= (uint32_t)(kWinBins - 1)) return;
-    uint32_t r0, r1;
-    block_regions(g, b, blockIdx.x, &r0, &r1);
-    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
-    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-    uint32_t* rpick = w.reg_pick + (uint64_t)b * g.regions;
-    uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
-    const int lane = threadIdx.x & (kWave - 1);
-    for (uint32_t s0 = r0 * kRegSlots; s0 < r1 * kRegSlots; s0 += kChunk * kBlock) {
-        const SlotChunk c = load_slots(rc, lb, s0, r1 * kRegSlots);
-        note_dense(c, dl);
-        uint32_t mine = 0;
-        bool hit[kChunk];
-#pragma unroll
-        for (int j = 0; j < kChunk; j++) {
-            const uint32_t bin = c.valid[j] ? window_bin(c.bits[j] & 0x7FFFFFFFu, lo, hi, shift) : 0u;
-            hit[j] = c.valid[j] && bin == jstar;
-            mine += hit[j] ? 1u : 0u;
-            const uint64_t above = __ballot(c.valid[j] && bin > jstar);  // a wavefront = one region
-            if (lane == 0 && c.region[j] < r1) rpick[c.region[j]] = (uint32_t)__popcll(above);
-        }
-        uint32_t total;
-        uint32_t pos = block_exclusive_scan(mine, scratch, &total);
-        if (total) {  // uniform
-            if (threadIdx.x == 0) gbase = atomicAdd(st + S_N2, total);
-            __syncthreads();
-            pos += gbase;
-#pragma unroll
-            for (int j = 0; j < kChunk; j++) {
-                if (hit[j]) {
-                    if (pos < g.lcap2) {
-                        l2[2 * (uint64_t)pos] = c.idx[j];
-                        l2[2 * (uint64_t)pos + 1] = c.bits[j] & 0x7FFFFFFFu;
-                    }
-                    pos++;
-                }
-            }
-            __syncthreads();
-        }
-    }
-    __syncthreads();
-    if (dl[0]) {  // rare
-        const uint64_t bn = bucket_count(g, b);
-        const float* rp = residual + (uint64_t)b * g.bucket_elems;
-        uint32_t cursor = threadIdx.x / kWave;
-        for (uint32_t r; (r = next_dense(dl, rc, &cursor, r0, r1)) != ~0u;) {
-            const uint64_t e0 = (uint64_t)r * kRegion;
-            const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
-            uint32_t above_total = 0;
-            uint32_t* buf = dreg[threadIdx.x / kWave];
-            stage_region(rp, e0, e1, buf);
-            for (uint64_t base = e0; base < e1; base += kWave) {  // wave-uniform trip count
-                const uint64_t i = base + lane;
-                const uint32_t key = i < e1 ? (buf[i - e0] & 0x7FFFFFFFu) : 0u;
-                const uint32_t bin = (i < e1 && key >= lo) ? window_bin(key, lo, hi, shift) : 0u;
-                const bool cand = i < e1 && key >= lo;
-                above_total += (uint32_t)__popcll(__ballot(cand && bin > jstar));
-                const uint64_t hm = __ballot(cand && bin == jstar);
-                if (hm) {
-                    uint32_t base2 = 0;
-                    if (lane == 0) base2 = atomicAdd(st + S_N2, (uint32_t)__popcll(hm));
-                    base2 = __shfl(base2, 0, kWave);
-                    if (cand && bin == jstar) {
-                        const uint32_t pos = base2 + (uint32_t)__popcll(hm & ((1ull << lane) - 1ull));
-                        if (pos < g.lcap2) {
-                            l2[2 * (uint64_t)pos] = (uint32_t)i;
-                            l2[2 * (uint64_t)pos + 1] = key;
-                        }
-                    }
-                }
-            }
-            if (lane == 0) rpick[r] = above_total;
-        }
-    }
-}
-
-// Whole exact selection of one bucket by one block: the fallback for buckets
-// whose candidate lists turned out incomplete.  Slow (one block streams the
-// bucket five times) but costs no extra launch: select2 calls it in place.
-// lh: kBins0 words, scratch: THREADS / kWave + 2 words of LDS.
-template <int THREADS>
-__device__ void bucket_exact(float* residual, const Geometry& g, uint32_t b, uint8_t* wire, uint64_t wire_stride,
-                             uint32_t* lh, uint32_t* scratch) {
-    const uint64_t bn = bucket_count(g, b);
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
-    uint32_t prefix = 0, remaining = bucket_k(g, b);
-    for (int round = 0; round < 3; round++) {
-        const int bins = round == 0 ? kBins0 : kBinsR;
-        const int shift = round == 0 ? 20 : (round == 1 ? 10 : 0);
-        const int hi_shift = round == 0 ? 31 : shift + 10;
-        for (int i = threadIdx.x; i < kBins0; i += THREADS) lh[i] = 0;
-        __syncthreads();
-        for (uint64_t i = threadIdx.x; i < bn; i += THREADS) {
-            const uint32_t key = key_of(rp[i]);
-            if ((key >> hi_shift) == (prefix >> hi_shift)) atomicAdd(&lh[(key >> shift) & (bins - 1)], 1u);
-        }
-        __syncthreads();
-        uint32_t left, bin;
-        if (round == 0) bin = pick_bin<kBins0, THREADS>(lh, remaining, 0, &left, scratch);
-        else bin = pick_bin<kBinsR, THREADS>(lh, remaining, 0, &left, scratch);
-        prefix |= bin << shift;
-        remaining = left;
-    }
-    const uint32_t T = prefix, need = remaining;
-    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
-    if (threadIdx.x == 0) out[0] = bucket_k(g, b);
-    uint32_t gt_run = 0, eq_run = 0;
-    for (uint64_t base = 0; base < bn; base += THREADS) {
-        const uint64_t i = base + threadIdx.x;
-        const uint32_t bitsv = i < bn ? f2u(rp[i]) : 0u;
-        const uint32_t key = bitsv & 0x7FFFFFFFu;
-        const bool is_gt = i < bn && key > T;
-        const bool is_eq = i < bn && key == T;
-        uint32_t total;
-        const uint32_t ex = block_exclusive_scan_n<THREADS>((is_gt ? 1u : 0u) + (is_eq ? 0x10000u : 0u), scratch,
-                                                                &total);
-        const uint32_t gt_b = gt_run + (ex & 0xFFFFu), eq_b = eq_run + (ex >> 16);
-        if (is_gt || (is_eq && eq_b < need)) {
-            const uint32_t pos = gt_b + (eq_b < need ? eq_b : need);
-            out[1 + 2 * (uint64_t)pos] = (uint32_t)i;
-            out[2 + 2 * (uint64_t)pos] = bitsv;
-            rp[i] = 0.0f;
-        }
-        gt_run += total & 0xFFFFu;
-        eq_run += total >> 16;
-    }
-}
-
-// Puts back the values pass A replaced by 0.0f (listed candidates with key >=
-// the predicted threshold) so that the exact fallback sees the plain sums.
-// Called by all threads of a select2 block.
-template <int THREADS>
-__device__ void restore_prezeroed(float* residual, const Geometry& g, const Workspace& w, uint32_t b) {
-    const uint32_t that_key = w.state[(uint64_t)b * kStateWords + S_THAT];
-    const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
-    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
-    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
-    for (uint32_t slot = threadIdx.x; slot < nreg * kRegSlots; slot += THREADS) {
-        const uint32_t cnt = rc[slot / kRegSlots];
-        if (cnt == kDense || (slot % kRegSlots) >= cnt) continue;
-        const uint32_t idx = lb[2 * (uint64_t)slot], bitsv = lb[2 * (uint64_t)slot + 1];
-        if ((bitsv & 0x7FFFFFFFu) >= that_key) rp[idx] = u2f(bitsv);
-    }
-    __threadfence();
-    __syncthreads();
-}
-
-// select, step 2: one block per bucket.  Checks that the threshold lies inside
-// the window and list2 is complete (else the bucket takes the exact fallback),
-// finishes the radix select on list2 (keys of one window bin: 24 bits at most
-// remain), resolves ties by index, adds the threshold bin's picks to the
-// per-region pick counts and turns those into each region's offset in the payload.
-__global__ __launch_bounds__(kSelThreads) void k_topk_select2(float* residual, Geometry g, Workspace w,
-                                                              uint8_t* wire, uint64_t wire_stride) {
-    __shared__ uint32_t lh[kBins0];
-    __shared__ uint32_t scratch[kSelThreads / kWave + 2];
-    const uint32_t b = blockIdx.x;
-    uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint32_t jstar = st[S_P0];
-    uint32_t want = st[S_R0];
-    const uint32_t count2 = st[S_N2];
-    if (jstar >= (uint32_t)(kWinBins - 1) || count2 > g.lcap2) {
-        // threshold outside the window, or more keys in its bin than list2 holds (rare):
-        // this block runs the whole exact selection of the bucket; S_OK stays 0, so emit skips it
-        restore_prezeroed<kSelThreads>(residual, g, w, b);
-        bucket_exact<kSelThreads>(residual, g, b, wire, wire_stride, lh, scratch);
-        return;
-    }
-
-    const uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
-    const uint32_t bin_lo = st[S_LO_KEY] + (jstar << st[S_SHIFT]);  // smallest key of the bin
-    uint32_t vprefix = 0;  // key - bin_lo: up to 30 bits, selected as 10 + 10 + 10
-    // a window bin spans 2^S_SHIFT keys: rounds whose digits lie wholly above that are skipped
-    const int first_round = st[S_SHIFT] <= 10 ? 2 : (st[S_SHIFT] <= 20 ? 1 : 0);
-    for (int r = first_round; r < 3; r++) {
-        const int shift = 20 - 10 * r;
-        const int hs = shift + 10;
-        for (int i = threadIdx.x; i < kBinsR; i += kSelThreads) lh[i] = 0;
-        __syncthreads();
-        for (uint32_t i = threadIdx.x; i < count2; i += kSelThreads) {
-            const uint32_t v = l2[2 * (uint64_t)i + 1] - bin_lo;
-            if ((v >> hs) == (vprefix >> hs)) atomicAdd(&lh[(v >> shift) & (kBinsR - 1)], 1u);
-        }
-        __syncthreads();
-        uint32_t left;
-        const uint32_t bin = pick_bin<kBinsR, kSelThreads>(lh, want, 0, &left, scratch);
-        vprefix |= bin << shift;
-        want = left;
-    }
-    const uint32_t T = bin_lo + vprefix;
-    const uint32_t need2 = want;
-    const uint32_t ties = lh[vprefix & (kBinsR - 1)];
-    __syncthreads();
-
-    // ties: when only some keys equal to T are taken, they are the `need2` lowest
-    // indices: radix-select the need2-th smallest index (11 + 11 + 10 bits)
-    uint32_t istar = 0xFFFFFFFFu;
-    if (ties != need2) {
-        uint32_t iwant = need2, iprefix = 0;
-        const int shifts[3] = {21, 10, 0};
-        const int widths[3] = {11, 11, 10};
-        for (int r = 0; r < 3; r++) {
-            const int bins = 1 << widths[r];
-            for (int i = threadIdx.x; i < kBins0; i += kSelThreads) lh[i] = 0;
-            __syncthreads();
-            const int hs = shifts[r] + widths[r];
-            for (uint32_t i = threadIdx.x; i < count2; i += kSelThreads) {
-                const uint32_t idx = l2[2 * (uint64_t)i], key = l2[2 * (uint64_t)i + 1];
-                const bool match = hs >= 32 ? true : ((idx >> hs) == (iprefix >> hs));
-                // bins stored reversed, so that pick_bin's top-down scan runs over ascending indices
-                if (key == T && match) atomicAdd(&lh[(bins - 1) - ((idx >> shifts[r]) & (bins - 1))], 1u);
-            }
-            __syncthreads();
-            uint32_t left, rb;
-            if (bins == kBins0) rb = pick_bin<kBins0, kSelThreads>(lh, iwant, 0, &left, scratch);
-            else rb = pick_bin<kBinsR, kSelThreads>(lh, iwant, 0, &left, scratch);
-            iprefix |= ((uint32_t)(bins - 1) - rb) << shifts[r];
-            iwant = left;
-        }
-        istar = iprefix;
-    }
-
-    // picks inside the threshold bin join their regions' counts; then an exclusive
-    // scan over the regions gives each region's first position in the payload
-    uint32_t* rpick = w.reg_pick + (uint64_t)b * g.regions;
-    for (uint32_t i = threadIdx.x; i < count2; i += kSelThreads) {
-        const uint32_t idx = l2[2 * (uint64_t)i], key = l2[2 * (uint64_t)i + 1];
-        if (key > T || (key == T && idx <= istar)) atomicAdd(&rpick[idx / kRegion], 1u);
-    }
-    __threadfence();
-    __syncthreads();
-    const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
-    const uint32_t per = (nreg + kSelThreads - 1) / kSelThreads;
-    const uint32_t first = threadIdx.x * per;
-    uint32_t* roff = w.reg_off + (uint64_t)b * g.regions;
-    uint32_t total;
-    constexpr uint32_t kHeld = 8;  // counts a thread keeps in registers between the two sweeps
-    if (per <= kHeld) {
-        uint32_t held[kHeld];
-#pragma unroll
-        for (uint32_t j = 0; j < kHeld; j++)
-            held[j] = (j < per && first + j < nreg)
-                          ? __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-        uint32_t sum = 0;
-#pragma unroll
-        for (uint32_t j = 0; j < kHeld; j++) sum += held[j];
-        uint32_t run = block_exclusive_scan_n<kSelThreads>(sum, scratch, &total);
-#pragma unroll
-        for (uint32_t j = 0; j < kHeld; j++) {
-            if (j < per && first + j < nreg) roff[first + j] = run;
-            run += held[j];
-        }
-    } else {
-        uint32_t sum = 0;
-        for (uint32_t j = 0; j < per; j++)
-            if (first + j < nreg) sum += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t run = block_exclusive_scan_n<kSelThreads>(sum, scratch, &total);
-        for (uint32_t j = 0; j < per; j++) {
-            if (first + j < nreg) {
-                roff[first + j] = run;
-                run += __hip_atomic_load(&rpick[first + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-    }
-    if (threadIdx.x == 0) {
-        st[S_T] = T;
-        st[S_NEED] = need2;
-        st[S_ISTAR] = istar;
-        st[S_OK] = total == bucket_k(g, b) ? 1u : 0u;
-    }
-    if (total != bucket_k(g, b)) {  // uniform; cannot happen with consistent lists
-        __syncthreads();
-        restore_prezeroed<kSelThreads>(residual, g, w, b);
-        bucket_exact<kSelThreads>(residual, g, b, wire, wire_stride, lh, scratch);
-    }
-}
-
-// Writes the payload: the picks of a region are its candidates with key > T, or
-// key == T and index <= istar, already in index order; they go to the region's
-// offset in pick order.  The residual already holds 0.0f where pass A predicted
-// a pick; picks it missed are zeroed and wrongly predicted ones get their value
-// back.  A wavefront handles one region at a time.
-__global__ __launch_bounds__(kBlock) void k_topk_emit_fast(float* residual, Geometry g, Workspace w, uint8_t* wire,
-                                                           uint64_t wire_stride) {
-    const uint32_t b = blockIdx.y;
-    const uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    if (!st[S_OK]) return;
-    const uint32_t T = st[S_T], istar = st[S_ISTAR], that_key = st[S_THAT];
-    uint32_t r0, r1;
-    block_regions(g, b, blockIdx.x, &r0, &r1);
-    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
-    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-    const uint32_t* roff = w.reg_off + (uint64_t)b * g.regions;
-    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
-    if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
-    const int lane = threadIdx.x & (kWave - 1);
-    __shared__ uint32_t dl[kDenseList + 2];
-    __shared__ uint32_t dreg[kBlock / kWave][kRegion];
-    if (threadIdx.x == 0) dl[0] = 0;
-    __syncthreads();
-    for (uint32_t s0 = r0 * kRegSlots; s0 < r1 * kRegSlots; s0 += kChunk * kBlock) {
-        uint32_t off[kChunk];
-#pragma unroll
-        for (int j = 0; j < kChunk; j++) {
-            const uint32_t r = (s0 + (uint32_t)j * kBlock + threadIdx.x) / kRegSlots;
-            off[j] = r < r1 ? roff[r] : 0u;
-        }
-        const SlotChunk c = load_slots(rc, lb, s0, r1 * kRegSlots);
-        note_dense(c, dl);
-#pragma unroll
-        for (int j = 0; j < kChunk; j++) {
-            const uint32_t key = c.bits[j] & 0x7FFFFFFFu;
-            const bool pick = c.valid[j] && (key > T || (key == T && c.idx[j] <= istar));
-            const uint64_t m = __ballot(pick);
-            if (pick) {
-                const uint32_t pos = off[j] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
-                u2a e = {c.idx[j], c.bits[j]};
-                *(u2a4*)(out + 1 + 2 * (uint64_t)pos) = e;
-            }
-            // pass A stored 0.0f for key >= predicted threshold; repair where the prediction was wrong
-            if (c.valid[j] && pick != (key >= that_key)) rp[c.idx[j]] = pick ? 0.0f : u2f(c.bits[j]);
-        }
-    }
-    __syncthreads();
-    if (dl[0]) {  // rare
-        const uint64_t bn = bucket_count(g, b);
-        uint32_t cursor = threadIdx.x / kWave;
-        for (uint32_t r; (r = next_dense(dl, rc, &cursor, r0, r1)) != ~0u;) {
-            const uint64_t e0 = (uint64_t)r * kRegion;
-            const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
-            uint32_t pos0 = roff[r];
-            uint32_t* buf = dreg[threadIdx.x / kWave];
-            stage_region(rp, e0, e1, buf);
-            for (uint64_t base = e0; base < e1; base += kWave) {  // wave-uniform trip count
-                const uint64_t i = base + lane;
-                const uint32_t bitsv = i < e1 ? buf[i - e0] : 0u;
-                const uint32_t key = bitsv & 0x7FFFFFFFu;
-                const bool pick = i < e1 && (key > T || (key == T && (uint32_t)i <= istar));
-                const uint64_t m = __ballot(pick);
-                if (pick) {
-                    const uint32_t pos = pos0 + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
-                    out[1 + 2 * (uint64_t)pos] = (uint32_t)i;
-                    out[2 + 2 * (uint64_t)pos] = bitsv;
-                    rp[i] = 0.0f;
-                }
-                pos0 += (uint32_t)__popcll(m);
-            }
-        }
-    }
-}
-
 // ================================ fused tail ======================================
 // Everything after the streaming pass in one launch: window histogram, threshold
 // bin, exact threshold, tie-break, payload offsets and the payload itself.  The
@@ -1258,6 +814,22 @@ __device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) {
 }
 __device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Histogram add called by all lanes of a wavefront (m: this lane has a key).  When all
+// keys of the wavefront fall into one bin - zeros, constants: the inputs that reach the
+// dense-region and exact paths - one lane adds the count; 64 adds to one LDS address
+// would serialise.
+__device__ __forceinline__ void wave_hist_add(uint32_t* lh, bool m, uint32_t bin) {
+    const uint64_t act = __ballot(m);
+    if (!act) return;
+    const int first = __ffsll((long long)act) - 1;
+    const uint32_t fb = (uint32_t)__shfl((int)bin, first, kWave);
+    if (__ballot(m && bin == fb) == act) {
+        if ((int)(threadIdx.x & (kWave - 1)) == first) atomicAdd(&lh[fb], (uint32_t)__popcll(act));
+    } else if (m) {
+        atomicAdd(&lh[bin], 1u);
+    }
 }
 
 // All threads of the block call it.  Returns false when the wait timed out.
@@ -1352,11 +924,153 @@ __device__ __forceinline__ uint32_t resolve_ties(const uint32_t* l2, uint32_t co
     return iprefix;
 }
 
-// The bucket goes to the exact selection (run by one block; S_OK stays 0).
-__device__ __forceinline__ void tail_fallback(float* residual, const Geometry& g, const Workspace& w, uint32_t b,
-                                           uint8_t* wire, uint64_t wire_stride, uint32_t* lh, uint32_t* scratch) {
-    restore_prezeroed<kBlock>(residual, g, w, b);
-    bucket_exact<kBlock>(residual, g, b, wire, wire_stride, lh, scratch);
+// The exact selection of one bucket by the kNSub blocks that work on it: the
+// fallback for a bucket whose window could not finish the selection (too few
+// candidates, threshold outside the window, a threshold bin with more keys than
+// list2 holds).  No extra launch; every block of the bucket enters it together.
+//   1  each block puts back, in its own regions, what the streaming pass stored as 0.0f
+//   2  three radix rounds over the key (11 + 10 + 10 bits): a block histograms its
+//      own slice of the bucket in LDS and adds it to the bucket's histogram; after
+//      a barrier every block scans that histogram and gets the same digit
+//   3  a block counts the keys above and at the threshold in its slice; after a
+//      barrier every block knows how many picks precede its slice
+//   4  a block writes its slice's picks in index order and zeroes them
+// A block only ever reads the residual range it restored itself, so the residual
+// needs no exchange between blocks.  lh: kBins0 words, scratch: kBlock / kWave + 2
+// words, flag: one word of LDS.  Returns false when a barrier wait timed out;
+// *T_out receives the exact threshold key.
+__device__ __forceinline__ bool bucket_exact_group(float* residual, const Geometry& g, const Workspace& w, uint32_t b, uint32_t s,
+                                   const Window& wn, uint8_t* wire, uint64_t wire_stride, uint32_t* lh,
+                                   uint32_t* scratch, uint32_t* flag, uint64_t limit_ticks, uint32_t* T_out) {
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    const uint64_t bn = bucket_count(g, b);
+    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    uint32_t r0, r1;
+    block_regions(g, b, s, &r0, &r1);
+    const uint64_t e0 = (uint64_t)r0 * kRegion;
+    const uint64_t e1 = (uint64_t)r1 * kRegion < bn ? (uint64_t)r1 * kRegion : bn;
+    // 1: this block's regions
+    {
+        const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
+        const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
+        for (uint32_t slot = r0 * kRegSlots + threadIdx.x; slot < r1 * kRegSlots; slot += kBlock) {
+            const uint32_t cnt = rc[slot / kRegSlots];
+            if (cnt == kDense || (slot % kRegSlots) >= cnt) continue;
+            const uint32_t idx = lb[2 * (uint64_t)slot], bitsv = lb[2 * (uint64_t)slot + 1];
+            if ((bitsv & 0x7FFFFFFFu) >= wn.that) rp[idx] = u2f(bitsv);
+        }
+        __syncthreads();
+    }
+    // 2: radix select.  Every wavefront walks a contiguous quarter of the block's slice,
+    // 64 elements per step with the loads of eight steps in flight; f(i, bits, valid) is
+    // called by all lanes of the wavefront for every step.
+    constexpr int NW = kBlock / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const uint64_t below = (1ull << lane) - 1ull;
+    const uint64_t quarter = ((e1 - e0 + NW - 1) / NW + kWave - 1) / kWave * kWave;
+    const uint64_t ws0 = e0 + (uint64_t)wave * quarter < e1 ? e0 + (uint64_t)wave * quarter : e1;
+    const uint64_t ws1 = ws0 + quarter < e1 ? ws0 + quarter : e1;
+    auto walk = [&](auto&& f) {
+        constexpr int B = 8;
+#pragma unroll 1
+        for (uint64_t base = ws0; base < ws1; base += (uint64_t)B * kWave) {
+            uint32_t v[B];
+#pragma unroll
+            for (int j = 0; j < B; j++) {
+                const uint64_t i = base + (uint64_t)j * kWave + lane;
+                v[j] = i < ws1 ? f2u(rp[i]) : 0u;
+            }
+#pragma unroll
+            for (int j = 0; j < B; j++) {
+                const uint64_t i = base + (uint64_t)j * kWave + lane;
+                if (base + (uint64_t)j * kWave < ws1) f(i, v[j], i < ws1);  // wave-uniform
+            }
+        }
+    };
+    uint32_t* gh = w.hist + (uint64_t)b * kHistWords;  // zero at kernel start
+    uint32_t prefix = 0, remaining = bucket_k(g, b);
+#pragma unroll 1
+    for (int round = 0; round < 3; round++) {
+        const int bins = round == 0 ? kBins0 : kBinsR;
+        const int shift = round == 0 ? 20 : (round == 1 ? 10 : 0);
+        const int hi_shift = round == 0 ? 31 : shift + 10;
+        uint32_t* ghr = gh + (round == 0 ? 0 : (round == 1 ? kBins0 : kBins0 + kBinsR));
+        for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
+        __syncthreads();
+        walk([&](uint64_t, uint32_t v, bool valid) {
+            const uint32_t key = v & 0x7FFFFFFFu;
+            wave_hist_add(lh, valid && (key >> hi_shift) == (prefix >> hi_shift), (key >> shift) & (uint32_t)(bins - 1));
+        });
+        __syncthreads();
+        for (int i = threadIdx.x; i < bins; i += kBlock) {
+            const uint32_t c = lh[i];
+            if (c) __hip_atomic_fetch_add(&ghr[i], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (!bucket_barrier(st + S_BARF + round, kNSub, flag, limit_ticks)) return false;
+        for (int i = threadIdx.x; i < bins; i += kBlock) lh[i] = ld_agent(&ghr[i]);
+        __syncthreads();
+        uint32_t left, bin;
+        if (round == 0) bin = pick_bin<kBins0, kBlock>(lh, remaining, 0, &left, scratch);
+        else bin = pick_bin<kBinsR, kBlock>(lh, remaining, 0, &left, scratch);
+        prefix |= bin << shift;
+        remaining = left;
+    }
+    const uint32_t T = prefix, need = remaining;
+    // 3: keys above and at the threshold per wavefront range, per block, and in the slices before
+    uint32_t gt_w = 0, eq_w = 0;  // wave-uniform
+    walk([&](uint64_t, uint32_t v, bool valid) {
+        const uint32_t key = v & 0x7FFFFFFFu;
+        gt_w += (uint32_t)__popcll(__ballot(valid && key > T));
+        eq_w += (uint32_t)__popcll(__ballot(valid && key == T));
+    });
+    uint32_t* wsum = lh;  // LDS words free again: [0..NW) above, [NW..2NW) equal
+    __syncthreads();
+    if (lane == 0) { wsum[wave] = gt_w; wsum[NW + wave] = eq_w; }
+    __syncthreads();
+    uint32_t gt_run = 0, eq_run = 0, gt_blk = 0, eq_blk = 0;
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+        if (i < wave) { gt_run += wsum[i]; eq_run += wsum[NW + i]; }
+        gt_blk += wsum[i];
+        eq_blk += wsum[NW + i];
+    }
+    if (threadIdx.x == 0) {
+        st_agent(&w.blk_above[(uint64_t)b * kNSub + s], gt_blk);
+        st_agent(&w.blk_eq[(uint64_t)b * kNSub + s], eq_blk);
+    }
+    if (!bucket_barrier(st + S_BARF + 3, kNSub, flag, limit_ticks)) return false;
+    {
+        static_assert(kNSub <= kBlock, "one thread per block of the bucket");
+        const uint32_t vg = threadIdx.x < s ? ld_agent(&w.blk_above[(uint64_t)b * kNSub + threadIdx.x]) : 0u;
+        const uint32_t ve = threadIdx.x < s ? ld_agent(&w.blk_eq[(uint64_t)b * kNSub + threadIdx.x]) : 0u;
+        uint32_t gt_before, eq_before;
+        block_exclusive_scan(vg, scratch, &gt_before);
+        block_exclusive_scan(ve, scratch, &eq_before);
+        gt_run += gt_before;
+        eq_run += eq_before;
+    }
+    // 4: this wavefront's picks, in index order: an element lands at (keys above T before it)
+    // + min(keys equal to T before it, need); ties are taken while fewer than need came before
+    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
+    if (s == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
+    walk([&](uint64_t i, uint32_t v, bool valid) {
+        const uint32_t key = v & 0x7FFFFFFFu;
+        const bool is_gt = valid && key > T, is_eq = valid && key == T;
+        const uint64_t mg = __ballot(is_gt), me = __ballot(is_eq);
+        const uint32_t gt_b = gt_run + (uint32_t)__popcll(mg & below);
+        const uint32_t eq_b = eq_run + (uint32_t)__popcll(me & below);
+        if (is_gt || (is_eq && eq_b < need)) {
+            const uint32_t pos = gt_b + (eq_b < need ? eq_b : need);
+            out[1 + 2 * (uint64_t)pos] = (uint32_t)i;
+            out[2 + 2 * (uint64_t)pos] = v;
+            rp[i] = 0.0f;
+        }
+        gt_run += (uint32_t)__popcll(mg);
+        eq_run += (uint32_t)__popcll(me);
+    });
+    *T_out = T;
+    return true;
 }
 
 __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geometry g, Workspace w, uint8_t* wire,
@@ -1369,7 +1083,8 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
     __shared__ uint32_t dbuf[NW][16 * kWave];  // dense_walk's staging area, one per wavefront
     const uint32_t b = blockIdx.y, s = blockIdx.x;
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint32_t lo = st[S_LO_KEY], hi = st[S_HI_KEY], shift = st[S_SHIFT], that_key = st[S_THAT];
+    const Window wn = load_window(st);
+    const uint32_t lo = wn.lo, hi = wn.hi, shift = wn.shift, that_key = wn.that;
     const uint32_t k = bucket_k(g, b);
     const uint64_t bn = bucket_count(g, b);
     uint32_t r0, r1;
@@ -1431,15 +1146,20 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
     bool failed = false;
 
     // ---- phase 1: window histogram -------------------------------------------------
+    // (A window that does not fit the histogram - only possible when the state words hold
+    // foreign contents - skips the work but not the barrier: a block that reaches the end
+    // of the kernel may rewrite the window, so every block must have read it by then.)
     for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
     __syncthreads();
+    if (wn.sound)
     sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t, uint32_t bitsv) {
               if ((uint32_t)lane < cnt) atomicAdd(&lh[window_bin(bitsv & 0x7FFFFFFFu, lo, hi, shift)], 1u);
           },
           [&](uint32_t, uint32_t r) {
               dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
                   const uint32_t key = v & 0x7FFFFFFFu;
-                  if (in && key >= lo) atomicAdd(&lh[window_bin(key, lo, hi, shift)], 1u);
+                  const bool cand = in && key >= lo;
+                  wave_hist_add(lh, cand, cand ? window_bin(key, lo, hi, shift) : 0u);
               });
           });
     __syncthreads();
@@ -1453,6 +1173,10 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
     }
 
     do {
+    if (!wn.sound) {
+        failed = true;
+        break;
+    }
     // ---- phase 2: threshold bin; certain picks per block; the bin's candidates to list2
     for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = ld_agent(&hw[i]);
     __syncthreads();
@@ -1670,10 +1394,18 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
         st[S_NEED] = need2;
         st[S_ISTAR] = istar;
         st[S_OK] = 1u;
+        predict_next_window(st, T);
     }
     } while (false);
-    // the exact selection for a bucket the window could not finish: one block runs it, S_OK stays 0
-    if (failed && s == 0) tail_fallback(residual, g, w, b, wire, wire_stride, lh, scratch);
+    // the exact selection for a bucket the window could not finish (S_OK stays 0)
+    if (failed) {
+        uint32_t T;
+        if (!bucket_exact_group(residual, g, w, b, s, wn, wire, wire_stride, lh, scratch, &sh_x[0], limit_ticks, &T)) {
+            if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
+            return;
+        }
+        if (s == 0 && threadIdx.x == 0) predict_next_window(st, T);
+    }
 }
 
 // ================================ host side =======================================
@@ -1687,9 +1419,9 @@ uint64_t zeroed_words(const Geometry& g) {
 
 uint64_t workspace_words(const Geometry& g) {
     return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) +
-           3 * align4((uint64_t)g.nbuckets * g.regions) +
+           align4((uint64_t)g.nbuckets * g.regions) +
            align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2) + align4((uint64_t)g.nbuckets * g.lcap2 * 2) +
-           align4((uint64_t)g.nbuckets * kNSub);
+           2 * align4((uint64_t)g.nbuckets * kNSub);
 }
 
 Workspace carve(void* base, const Geometry& g) {
@@ -1701,11 +1433,10 @@ Workspace carve(void* base, const Geometry& g) {
     w.tile_gt = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
     w.tile_eq = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
     w.reg_cnt = p;     p += align4((uint64_t)g.nbuckets * g.regions);
-    w.reg_pick = p;    p += align4((uint64_t)g.nbuckets * g.regions);
-    w.reg_off = p;     p += align4((uint64_t)g.nbuckets * g.regions);
     w.list = p;        p += align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2);
     w.list2 = p;       p += align4((uint64_t)g.nbuckets * g.lcap2 * 2);
-    w.blk_above = p;
+    w.blk_above = p;   p += align4((uint64_t)g.nbuckets * kNSub);
+    w.blk_eq = p;
     return w;
 }
 
@@ -1730,12 +1461,48 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     return true;
 }
 
+// Workspaces whose state words hold a window prediction: address -> shape of the last
+// single-pass call that used it.  A call finds its workspace here with the same shape
+// and skips the sample kernel; anything else (first use, another shape, the exact path
+// in between, mccl_hip_topk_workspace_forget) starts from a fresh sample.
+struct WarmShape {
+    uint64_t n_total, bucket_elems;
+    double ratio;
+    int device;
+};
+std::mutex g_warm_mu;
+std::unordered_map<uintptr_t, WarmShape> g_warm;
+
+bool take_warm(void* workspace, const Geometry& g, double ratio, bool single_pass) {
+    std::lock_guard<std::mutex> lock(g_warm_mu);
+    const uintptr_t key = (uintptr_t)workspace;
+    if (!single_pass) {
+        g_warm.erase(key);
+        return false;
+    }
+    const WarmShape now = {g.n_total, g.bucket_elems, ratio, device_info().device};
+    auto it = g_warm.find(key);
+    const bool warm = it != g_warm.end() && it->second.n_total == now.n_total &&
+                      it->second.bucket_elems == now.bucket_elems && it->second.ratio == now.ratio &&
+                      it->second.device == now.device;
+    if (g_warm.size() > 4096 && it == g_warm.end()) g_warm.clear();
+    g_warm[key] = now;
+    return warm;
+}
+
 }  // namespace
 }  // namespace mcclhip
 
 using namespace mcclhip;
 
 extern "C" {
+
+int mccl_hip_topk_workspace_forget(void* workspace) {
+    if (!workspace) return MCCL_HIP_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_warm_mu);
+    g_warm.erase((uintptr_t)workspace);
+    return MCCL_HIP_OK;
+}
 
 uint32_t mccl_hip_topk_k(uint64_t count, double ratio) {
     uint32_t k = static_cast<uint32_t>(static_cast<double>(count) * ratio);
@@ -1782,22 +1549,15 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     const uint64_t need_r = (nvec + kBlock * 4 - 1) / (kBlock * 4);
     const uint32_t bx_r = clamp_u32(bx < need_r ? bx : need_r, 1, 65535);
     const uint32_t bx_t = clamp_u32(bx < g.tiles ? bx : g.tiles, 1, 65535);
+    const bool warm = take_warm(workspace, g, ratio, fast) && tuning().topk_warm != 0;
     if (fast) {
-        k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(grad, residual, g, w);
+        // the window comes from the previous call's exact threshold when there was one
+        if (!warm) k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(grad, residual, g, w);
         const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
         k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
-        if (tuning().topk_tail == 0) {
-            // 100 MHz ticks a block may wait at a barrier before it gives up
-            const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
-            k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride,
-                                                                    limit);
-        } else {
-            k_topk_window_hist<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
-            k_topk_select1<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w);
-            k_topk_select2<<<g.nbuckets, kSelThreads, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride);
-            k_topk_emit_fast<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire,
-                                                                         wire_stride);
-        }
+        // 100 MHz ticks a block may wait at a barrier before it gives up
+        const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
+        k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride, limit);
     } else {
         const uint64_t zw = zeroed_words(g);
         k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);

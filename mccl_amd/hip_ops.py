@@ -114,7 +114,10 @@ def topk_workspace(n_total: int, bucket_elems: int, ratio: float, device) -> tor
     nbytes = int(_lib.load().mccl_hip_topk_workspace_bytes(n_total, bucket_elems, ratio))
     if nbytes == 0:
         raise _lib.MCCLHipError(-6, "topk_workspace_bytes")
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    # the allocator may hand out an address an earlier workspace lived at
+    _lib.load().mccl_hip_topk_workspace_forget(ws.data_ptr())
+    return ws
 
 
 def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
@@ -141,6 +144,11 @@ def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
                                            workspace.numel(), _stream())
     _lib.check(rc, "topk_compress")
     return wire, stride
+
+
+def topk_workspace_forget(workspace: torch.Tensor) -> None:
+    """The next compress call with this workspace samples the gradient afresh."""
+    _lib.check(_lib.load().mccl_hip_topk_workspace_forget(workspace.data_ptr()), "topk_workspace_forget")
 
 
 def topk_path_report(workspace: torch.Tensor, n_total: int, bucket_elems: int, ratio: float):
