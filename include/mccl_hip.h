@@ -163,6 +163,24 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
                            uint64_t wire_stride, void* workspace, uint64_t workspace_bytes,
                            void* stream);
 
+/* TopKCompressor::compress for a LIST of buckets that are separate buffers of
+ * their own lengths (the tensor list of a coalesced allreduce,
+ * csrc/backend/ProcessGroupMCCL.cpp:2257-2313, compresses bucket by bucket), in
+ * the same three launches as mccl_hip_topk_compress: per-bucket calls are bound
+ * by launch latency, a list is not.  host_grads[b] / host_residuals[b] hold
+ * host_counts[b] fp32 elements; bucket b's payload [u32 k_b][k_b x {u32 index,
+ * f32 value}] goes to host_wires[b], which holds host_wire_capacities[b] bytes
+ * (at least 4 + 8 * k_b, else MCCL_HIP_ERR_CAPACITY; 4-byte aligned).  At most
+ * MCCL_HIP_TOPK_LIST_MAX buckets per call.  The host arrays are read before the
+ * call returns.  Results are identical to one mccl_hip_topk_compress call per
+ * bucket. */
+#define MCCL_HIP_TOPK_LIST_MAX 64
+uint64_t mccl_hip_topk_list_workspace_bytes(const uint64_t* host_counts, uint32_t nbuckets, double ratio);
+int mccl_hip_topk_compress_list(const float* const* host_grads, float* const* host_residuals,
+                                const uint64_t* host_counts, void* const* host_wires,
+                                const uint64_t* host_wire_capacities, uint32_t nbuckets, double ratio,
+                                void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* The workspace carries state from one call to the next: after a call it holds,
  * per bucket, the exact threshold just found, and the next call with the same
  * workspace and shape starts from it instead of sampling the gradient again (a

@@ -2,6 +2,8 @@
 
 #include <c10/hip/HIPStream.h>
 
+#include <algorithm>
+
 #include "../../../include/mccl_hip.h"
 #include <hip/hip_runtime_api.h>
 
@@ -9,6 +11,7 @@
 #include "FP16Compression.hpp"
 #include "HipKernels.hpp"
 #include "Logging.hpp"
+#include "TensorChecks.hpp"
 #include "TopKCompression.hpp"
 
 namespace mccl {
@@ -71,20 +74,12 @@ TopKCompressor::TopKCompressor(double k_ratio) : k_ratio_(k_ratio) {
     MCCL_CHECK(k_ratio > 0 && k_ratio <= 1.0, "k_ratio must be in (0, 1], got " + std::to_string(k_ratio));
 }
 
-// csrc/compression/TopKCompression.cpp:38-120.  The residual map keeps the
-// reference's rules: a new id while 1024 ids are live clears the map (:57-62);
-// an id whose element count changed starts again from zeros (:63-66).
-size_t TopKCompressor::compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
-                                at::ScalarType dtype, uint64_t stable_id) {
-    MCCL_CHECK(dtype == at::kFloat, "TopK compression currently supports float32 only");
-    const size_t count = nbytes / sizeof(float);
-    MCCL_CHECK(count > 0, "TopK compress: empty input");
-    const uint32_t k = mccl_hip_topk_k(count, k_ratio_);
-    const size_t output_size = sizeof(uint32_t) + static_cast<size_t>(k) * 8;
-    MCCL_CHECK(dst_capacity >= output_size, "TopK compress: buffer too small");
+TopKCompressor::~TopKCompressor() = default;
 
-    std::lock_guard<std::mutex> lock(mu_);
-    metal_kernels_init();
+// The residual map keeps the reference's rules (csrc/compression/TopKCompression.cpp:57-67):
+// a new id while 1024 ids are live clears the map; an id whose element count changed starts
+// again from zeros.  Caller holds mu_.
+at::Tensor& TopKCompressor::residual_for(uint64_t stable_id, size_t count) {
     const auto opts_f = at::TensorOptions().dtype(at::kFloat).device(at::kCUDA);
     if (error_buffers_.size() >= kMaxErrorBuffers && error_buffers_.find(stable_id) == error_buffers_.end()) {
         MCCL_WARN("TopK: evicting all %zu error feedback buffers (unstable tensor identities?)",
@@ -95,23 +90,104 @@ size_t TopKCompressor::compress(const void* src, size_t nbytes, void* dst, size_
     if (it == error_buffers_.end() || static_cast<size_t>(it->second.numel()) != count) {
         error_buffers_[stable_id] = at::zeros({static_cast<int64_t>(count)}, opts_f);
     }
-    at::Tensor& residual = error_buffers_[stable_id];
+    return error_buffers_[stable_id];
+}
 
+// One bucket on `stream`: csrc/compression/TopKCompression.cpp:38-120.  Caller holds mu_.
+size_t TopKCompressor::compress_on(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
+                                   at::Tensor& residual, at::Tensor& workspace, void* stream) {
+    const size_t count = nbytes / sizeof(float);
+    const uint32_t k = mccl_hip_topk_k(count, k_ratio_);
+    const size_t output_size = sizeof(uint32_t) + static_cast<size_t>(k) * 8;
     const uint64_t ws_bytes = mccl_hip_topk_workspace_bytes(count, count, k_ratio_);
-    if (!workspace_.defined() || static_cast<uint64_t>(workspace_.numel()) < ws_bytes) {
-        workspace_ = at::empty({static_cast<int64_t>(ws_bytes)},
-                               at::TensorOptions().dtype(at::kByte).device(at::kCUDA));
+    if (!workspace.defined() || static_cast<uint64_t>(workspace.numel()) < ws_bytes) {
+        workspace = at::empty({static_cast<int64_t>(ws_bytes)},
+                              at::TensorOptions().dtype(at::kByte).device(at::kCUDA));
     }
+    // the scratch is shared by buckets of different tensors: no threshold carried between calls
+    mccl_hip_topk_workspace_forget(workspace.data_ptr());
     // The payload's pairs start 4 bytes in; the stride only has to be a multiple of 4.
     const uint64_t stride = static_cast<uint64_t>(dst_capacity) & ~uint64_t(3);
     const int rc = mccl_hip_topk_compress(static_cast<const float*>(src), residual.data_ptr<float>(), count,
-                                          count, k_ratio_, dst, stride, workspace_.data_ptr(),
-                                          static_cast<uint64_t>(workspace_.numel()),
-                                          c10::hip::getCurrentHIPStream().stream());
+                                          count, k_ratio_, dst, stride, workspace.data_ptr(),
+                                          static_cast<uint64_t>(workspace.numel()), stream);
     if (rc == MCCL_HIP_ERR_CAPACITY) throw MCCLError("TopK compress: buffer too small");
     throw_on_status(rc, "TopK compress");
     MCCL_TRACE("TopK compress: %zu elements -> %u values, output %zu bytes", count, k, output_size);
     return output_size;
+}
+
+size_t TopKCompressor::compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
+                                at::ScalarType dtype, uint64_t stable_id) {
+    MCCL_CHECK(dtype == at::kFloat, "TopK compression currently supports float32 only");
+    const size_t count = nbytes / sizeof(float);
+    MCCL_CHECK(count > 0, "TopK compress: empty input");
+    const uint32_t k = mccl_hip_topk_k(count, k_ratio_);
+    MCCL_CHECK(dst_capacity >= sizeof(uint32_t) + static_cast<size_t>(k) * 8, "TopK compress: buffer too small");
+    std::lock_guard<std::mutex> lock(mu_);
+    metal_kernels_init();
+    at::Tensor& residual = residual_for(stable_id, count);
+    return compress_on(src, nbytes, dst, dst_capacity, residual, workspace_,
+                       c10::hip::getCurrentHIPStream().stream());
+}
+
+std::vector<at::Tensor> TopKCompressor::compress_many(const std::vector<at::Tensor>& buckets,
+                                                      const std::vector<uint64_t>& stable_ids) {
+    MCCL_CHECK(buckets.size() == stable_ids.size(), "compress_many: one stable id per bucket");
+    std::vector<at::Tensor> payloads;
+    if (buckets.empty()) return payloads;
+    std::lock_guard<std::mutex> lock(mu_);
+    metal_kernels_init();
+    std::vector<at::Tensor*> residuals;
+    for (size_t i = 0; i < buckets.size(); i++) {
+        const at::Tensor& t = buckets[i];
+        check_single_tensor(t);
+        MCCL_CHECK(t.scalar_type() == at::kFloat, "TopK compression currently supports float32 only");
+        MCCL_CHECK(t.numel() > 0, "TopK compress: empty input");
+        for (size_t j = 0; j < i; j++)
+            MCCL_CHECK(stable_ids[j] != stable_ids[i], "compress_many: the same stable id twice in one call");
+        payloads.push_back(at::empty({static_cast<int64_t>(max_compressed_size(tensor_nbytes(t)))},
+                                     at::TensorOptions().dtype(at::kByte).device(t.device())));
+    }
+    // (a second loop: residual_for may clear the map when the 1025th id arrives, and the
+    // references it returned before that would dangle)
+    for (size_t i = 0; i < buckets.size(); i++) residual_for(stable_ids[i], static_cast<size_t>(buckets[i].numel()));
+    for (size_t i = 0; i < buckets.size(); i++) {
+        auto it = error_buffers_.find(stable_ids[i]);
+        MCCL_CHECK(it != error_buffers_.end() && it->second.numel() == buckets[i].numel(),
+                   "compress_many: more distinct stable ids than the compressor holds residuals for");
+        residuals.push_back(&it->second);
+    }
+    // the list goes to the library in chunks of MCCL_HIP_TOPK_LIST_MAX buckets: three launches per chunk
+    const int device = buckets[0].get_device();
+    void* stream = c10::hip::getCurrentHIPStream(device).stream();
+    std::vector<size_t> used(buckets.size());
+    for (size_t first = 0; first < buckets.size(); first += MCCL_HIP_TOPK_LIST_MAX) {
+        const size_t n = std::min<size_t>(MCCL_HIP_TOPK_LIST_MAX, buckets.size() - first);
+        std::vector<const float*> grads(n);
+        std::vector<float*> res(n);
+        std::vector<uint64_t> counts(n), caps(n);
+        std::vector<void*> wires(n);
+        for (size_t i = 0; i < n; i++) {
+            grads[i] = buckets[first + i].data_ptr<float>();
+            res[i] = residuals[first + i]->data_ptr<float>();
+            counts[i] = static_cast<uint64_t>(buckets[first + i].numel());
+            wires[i] = payloads[first + i].data_ptr();
+            caps[i] = static_cast<uint64_t>(payloads[first + i].numel());
+            used[first + i] = sizeof(uint32_t) + static_cast<size_t>(mccl_hip_topk_k(counts[i], k_ratio_)) * 8;
+        }
+        const uint64_t need = mccl_hip_topk_list_workspace_bytes(counts.data(), static_cast<uint32_t>(n), k_ratio_);
+        if (!list_workspace_.defined() || static_cast<uint64_t>(list_workspace_.numel()) < need)
+            list_workspace_ = at::empty({static_cast<int64_t>(need)},
+                                        at::TensorOptions().dtype(at::kByte).device(at::kCUDA));
+        const int rc = mccl_hip_topk_compress_list(grads.data(), res.data(), counts.data(), wires.data(), caps.data(),
+                                                   static_cast<uint32_t>(n), k_ratio_, list_workspace_.data_ptr(),
+                                                   static_cast<uint64_t>(list_workspace_.numel()), stream);
+        if (rc == MCCL_HIP_ERR_CAPACITY) throw MCCLError("TopK compress: buffer too small");
+        throw_on_status(rc, "TopK compress");
+    }
+    for (size_t i = 0; i < buckets.size(); i++) payloads[i] = payloads[i].narrow(0, 0, static_cast<int64_t>(used[i]));
+    return payloads;
 }
 
 // csrc/compression/TopKCompression.cpp:122-152.  The reference validates while

@@ -243,6 +243,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             c.decompress(wire.data_ptr(), sz, out.data_ptr(), static_cast<size_t>(numel) * 4, at::kFloat);
             return out;
         }, py::arg("wire"), py::arg("numel"), py::arg("compressed_size") = py::none())
+        .def("compress_many", [](mccl::TopKCompressor& c, const std::vector<at::Tensor>& buckets, py::object stable_ids) {
+            std::vector<uint64_t> ids;
+            if (stable_ids.is_none()) for (const auto& t : buckets) ids.push_back(stable_id_of(t));
+            else ids = stable_ids.cast<std::vector<uint64_t>>();
+            return c.compress_many(buckets, ids);
+        }, py::arg("buckets"), py::arg("stable_ids") = py::none(),
+           "Top-k payloads of a list of gradient buckets, one uint8 device tensor each")
         .def("reset_error_feedback", &mccl::TopKCompressor::reset_error_feedback)
         .def("reset_error_feedback_for_tensor", &mccl::TopKCompressor::reset_error_feedback_for_tensor)
         .def("error_feedback_buffer_count", &mccl::TopKCompressor::error_feedback_buffer_count)

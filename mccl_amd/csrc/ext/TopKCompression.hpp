@@ -5,6 +5,7 @@
 
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "Compression.hpp"
 
@@ -13,6 +14,7 @@ namespace mccl {
 class TopKCompressor : public Compressor {
 public:
     explicit TopKCompressor(double k_ratio);
+    ~TopKCompressor() override;
 
     size_t compress(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
                     at::ScalarType dtype, uint64_t stable_id = 0) override;
@@ -29,6 +31,15 @@ public:
     /// checkpointing and tests.
     at::Tensor error_feedback_buffer(uint64_t stable_id) const;
 
+    /// compress() for a list of buckets (float32 device tensors, one stable id each), the shape
+    /// of a coalesced allreduce (csrc/backend/ProcessGroupMCCL.cpp:2257-2313 walks its tensor
+    /// list bucket by bucket).  Returns one payload tensor per bucket, identical to what the
+    /// per-bucket calls give.  A bucket's three launches are latency-bound (and fifteen calls
+    /// are bound by the host's launch rate), so the whole list goes through the same three
+    /// launches (mccl_hip_topk_compress_list).
+    std::vector<at::Tensor> compress_many(const std::vector<at::Tensor>& buckets,
+                                          const std::vector<uint64_t>& stable_ids);
+
     double k_ratio() const { return k_ratio_; }
 
 private:
@@ -36,8 +47,12 @@ private:
     mutable std::mutex mu_;
     // stable id -> fp32 residual in HBM, one element per gradient element
     std::unordered_map<uint64_t, at::Tensor> error_buffers_;
-    at::Tensor workspace_;
+    at::Tensor workspace_;       // scratch of a one-bucket call
+    at::Tensor list_workspace_;  // scratch of a list call
     at::Tensor status_;  // device int32[1], written by decompress
+    at::Tensor& residual_for(uint64_t stable_id, size_t count);
+    size_t compress_on(const void* src, size_t nbytes, void* dst, size_t dst_capacity, at::Tensor& residual,
+                       at::Tensor& workspace, void* stream);
     static constexpr size_t kMaxErrorBuffers = 1024;
 };
 

@@ -141,6 +141,7 @@ struct Geometry {
     uint32_t k_last;   // k of the last bucket
     uint32_t regions;  // fast path: candidate regions allotted per bucket
     uint32_t lcap2;    // fast path: capacity of a bucket's list2 (entries)
+    uint32_t listed;   // fast path: 1 when the buckets are separate buffers (see Buckets)
 };
 
 struct Workspace {
@@ -167,6 +168,45 @@ __device__ __forceinline__ uint32_t bucket_k(const Geometry& g, uint32_t b) {
     return b + 1 == g.nbuckets ? g.k_last : g.k_full;
 }
 __device__ __forceinline__ uint32_t key_of(float v) { return f2u(v) & 0x7FFFFFFFu; }
+
+// Where the buckets of a single-pass call live.  Uniform layout: the buckets are
+// consecutive ranges of one gradient (mccl_hip_topk_compress).  Listed layout
+// (Geometry::listed): every bucket is a buffer of its own with its own length
+// (mccl_hip_topk_compress_list); g.bucket_elems is then the longest bucket.
+constexpr uint32_t kMaxListed = MCCL_HIP_TOPK_LIST_MAX;
+struct Buckets {
+    const float* grad;
+    float* residual;
+    uint8_t* wire;
+    uint64_t wire_stride;
+    const float* lgrad[kMaxListed];
+    float* lresidual[kMaxListed];
+    uint8_t* lwire[kMaxListed];
+    uint32_t lcount[kMaxListed];
+    uint32_t lk[kMaxListed];
+};
+// The kernels index the table by bucket number.  Indexing the by-value parameter would make
+// the compiler copy all of it to per-lane scratch memory first (2 KiB per lane, and a launch
+// that sets up scratch starts several microseconds later); the kernels read it where it
+// already lies instead, in the kernel-argument segment, through scalar loads.  Buckets is
+// therefore the FIRST parameter of every kernel that takes one.
+typedef const __attribute__((address_space(4))) Buckets* BucketsArg;
+__device__ __forceinline__ BucketsArg buckets_arg() { return (BucketsArg)__builtin_amdgcn_kernarg_segment_ptr(); }
+__device__ __forceinline__ uint64_t bucket_count(const Geometry& g, BucketsArg bk, uint32_t b) {
+    return g.listed ? (uint64_t)bk->lcount[b] : bucket_count(g, b);
+}
+__device__ __forceinline__ uint32_t bucket_k(const Geometry& g, BucketsArg bk, uint32_t b) {
+    return g.listed ? bk->lk[b] : bucket_k(g, b);
+}
+__device__ __forceinline__ const float* bucket_grad(const Geometry& g, BucketsArg bk, uint32_t b) {
+    return g.listed ? bk->lgrad[b] : bk->grad + (uint64_t)b * g.bucket_elems;
+}
+__device__ __forceinline__ float* bucket_residual(const Geometry& g, BucketsArg bk, uint32_t b) {
+    return g.listed ? bk->lresidual[b] : bk->residual + (uint64_t)b * g.bucket_elems;
+}
+__device__ __forceinline__ uint32_t* bucket_wire(const Geometry& g, BucketsArg bk, uint32_t b) {
+    return (uint32_t*)(g.listed ? bk->lwire[b] : bk->wire + (uint64_t)b * bk->wire_stride);
+}
 
 __global__ __launch_bounds__(kBlock) void k_zero_words(uint32_t* p, uint64_t n) {
     // n is a multiple of 4 and p is 16-byte aligned (see carve())
@@ -536,16 +576,15 @@ __device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32
 //     r_hi = ks - 6 sqrt(ks) - 16,   r_lo = ks + 6 sqrt(ks) + 16   and   ks,
 // ks = k * S / n being the expected number of sampled elements among the top k:
 // the two ends of the candidate window and the predicted threshold.
-__global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __restrict__ grad,
-                                                             const float* __restrict__ residual, Geometry g,
-                                                             Workspace w) {
+__global__ __launch_bounds__(kSampleThreads) void k_topk_sample(Buckets, Geometry g, Workspace w) {
+    const BucketsArg bk = buckets_arg();
     __shared__ uint32_t keys[kSample];
     __shared__ uint32_t lh[3][kBinsR];
     __shared__ uint32_t scratch[3 * (kSampleThreads / kWave + 2)];
     const uint32_t b = blockIdx.x;
-    const uint64_t bn = bucket_count(g, b);
-    const float* gp = grad + (uint64_t)b * g.bucket_elems;
-    const float* rp = residual + (uint64_t)b * g.bucket_elems;
+    const uint64_t bn = bucket_count(g, bk, b);
+    const float* gp = bucket_grad(g, bk, b);
+    const float* rp = bucket_residual(g, bk, b);
     const uint64_t nvec = bn / 4;
     constexpr int SV = kSample / 4;  // sampled vectors
     // sampled in runs of 8 vectors (one 128-byte line per array), runs evenly spread
@@ -567,7 +606,7 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __r
         for (int q = 0; q < 4; q++) keys[4 * i + q] = i < nsv ? key_of(u2f(gv[j][q]) + u2f(rv[j][q])) : 0u;
     }
     const uint32_t S = nsv * 4;
-    const float ks = (float)bucket_k(g, b) * (float)S / (float)bn;
+    const float ks = (float)bucket_k(g, bk, b) * (float)S / (float)bn;
     const float margin = 6.0f * sqrtf(ks) + 16.0f;
     // ranks: 0 upper end of the window, 1 lower end, 2 the predicted threshold itself
     constexpr int NR = 3;
@@ -646,8 +685,9 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(const float* __r
 // atomics and no shared capacity are involved, so nothing can overflow.
 
 // The regions [r0, r1) of bucket b that block s of kNSub works on.
-__device__ __forceinline__ void block_regions(const Geometry& g, uint32_t b, uint32_t s, uint32_t* r0, uint32_t* r1) {
-    const uint32_t nreg = (uint32_t)((bucket_count(g, b) + kRegion - 1) / kRegion);
+__device__ __forceinline__ void block_regions(const Geometry& g, BucketsArg bk, uint32_t b, uint32_t s,
+                                              uint32_t* r0, uint32_t* r1) {
+    const uint32_t nreg = (uint32_t)((bucket_count(g, bk, b) + kRegion - 1) / kRegion);
     const uint32_t per = (nreg + kNSub - 1) / kNSub;
     *r0 = s * per < nreg ? s * per : nreg;
     *r1 = *r0 + per < nreg ? *r0 + per : nreg;
@@ -664,11 +704,11 @@ __device__ __forceinline__ void block_regions(const Geometry& g, uint32_t b, uin
 // Nothing else happens here: returning atomics and histogram flushes in these
 // 12,000 streaming blocks each cost 7-15 % of the kernel's time when they were
 // tried.
-__global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __restrict__ grad, float* residual,
-                                                             Geometry g, Workspace w) {
+__global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(Buckets, Geometry g, Workspace w) {
+    const BucketsArg bk = buckets_arg();
     __shared__ uint32_t stage[kBlock / kWave][kRegSlots][2];
     const uint32_t b = blockIdx.y, t = blockIdx.x;
-    const uint64_t bn = bucket_count(g, b);
+    const uint64_t bn = bucket_count(g, bk, b);
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const uint64_t w0 = (uint64_t)t * kATile + (uint64_t)wave * kRegion;  // first element of this wave's region
@@ -684,8 +724,8 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
         for (int i = threadIdx.x; i < kHistWords; i += kBlock) w.hist[(uint64_t)b * kHistWords + i] = 0;
     }
     if (w0 >= bn) return;  // whole wavefront; the kernel has no barriers
-    const float* gp = grad + (uint64_t)b * g.bucket_elems + w0;
-    float* rp = residual + (uint64_t)b * g.bucket_elems + w0;
+    const float* gp = bucket_grad(g, bk, b) + w0;
+    float* rp = bucket_residual(g, bk, b) + w0;
     constexpr int U = 2;
     constexpr int ROUNDS = kRegion / (kWave * 4 * U);
     const uint32_t len = (uint32_t)((bn - w0) < (uint64_t)kRegion ? (bn - w0) : (uint64_t)kRegion);
@@ -731,7 +771,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(const float* __rest
             // they reached the predicted threshold; put those values back
             dense = true;
             if ((uint32_t)lane < staged && (stage[wave][lane][1] & 0x7FFFFFFFu) >= that_key)
-                residual[(uint64_t)b * g.bucket_elems + stage[wave][lane][0]] = u2f(stage[wave][lane][1]);
+                bucket_residual(g, bk, b)[stage[wave][lane][0]] = u2f(stage[wave][lane][1]);
             return;
         }
         uint32_t pos = staged + before;
@@ -939,14 +979,15 @@ __device__ __forceinline__ uint32_t resolve_ties(const uint32_t* l2, uint32_t co
 // needs no exchange between blocks.  lh: kBins0 words, scratch: kBlock / kWave + 2
 // words, flag: one word of LDS.  Returns false when a barrier wait timed out;
 // *T_out receives the exact threshold key.
-__device__ __forceinline__ bool bucket_exact_group(float* residual, const Geometry& g, const Workspace& w, uint32_t b, uint32_t s,
-                                   const Window& wn, uint8_t* wire, uint64_t wire_stride, uint32_t* lh,
-                                   uint32_t* scratch, uint32_t* flag, uint64_t limit_ticks, uint32_t* T_out) {
+__device__ __forceinline__ bool bucket_exact_group(BucketsArg bk, const Geometry& g, const Workspace& w,
+                                                   uint32_t b, uint32_t s, const Window& wn, uint32_t* lh,
+                                                   uint32_t* scratch, uint32_t* flag, uint64_t limit_ticks,
+                                                   uint32_t* T_out) {
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint64_t bn = bucket_count(g, b);
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    const uint64_t bn = bucket_count(g, bk, b);
+    float* rp = bucket_residual(g, bk, b);
     uint32_t r0, r1;
-    block_regions(g, b, s, &r0, &r1);
+    block_regions(g, bk, b, s, &r0, &r1);
     const uint64_t e0 = (uint64_t)r0 * kRegion;
     const uint64_t e1 = (uint64_t)r1 * kRegion < bn ? (uint64_t)r1 * kRegion : bn;
     // 1: this block's regions
@@ -989,7 +1030,7 @@ __device__ __forceinline__ bool bucket_exact_group(float* residual, const Geomet
         }
     };
     uint32_t* gh = w.hist + (uint64_t)b * kHistWords;  // zero at kernel start
-    uint32_t prefix = 0, remaining = bucket_k(g, b);
+    uint32_t prefix = 0, remaining = bucket_k(g, bk, b);
 #pragma unroll 1
     for (int round = 0; round < 3; round++) {
         const int bins = round == 0 ? kBins0 : kBinsR;
@@ -1052,8 +1093,8 @@ __device__ __forceinline__ bool bucket_exact_group(float* residual, const Geomet
     }
     // 4: this wavefront's picks, in index order: an element lands at (keys above T before it)
     // + min(keys equal to T before it, need); ties are taken while fewer than need came before
-    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
-    if (s == 0 && threadIdx.x == 0) out[0] = bucket_k(g, b);
+    uint32_t* out = bucket_wire(g, bk, b);
+    if (s == 0 && threadIdx.x == 0) out[0] = bucket_k(g, bk, b);
     walk([&](uint64_t i, uint32_t v, bool valid) {
         const uint32_t key = v & 0x7FFFFFFFu;
         const bool is_gt = valid && key > T, is_eq = valid && key == T;
@@ -1073,8 +1114,8 @@ __device__ __forceinline__ bool bucket_exact_group(float* residual, const Geomet
     return true;
 }
 
-__global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geometry g, Workspace w, uint8_t* wire,
-                                                         uint64_t wire_stride, uint64_t limit_ticks) {
+__global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Workspace w, uint64_t limit_ticks) {
+    const BucketsArg bk = buckets_arg();
     constexpr int NW = kBlock / kWave;
     __shared__ uint32_t lh[kBins0];
     __shared__ uint32_t scratch[NW + 2];
@@ -1085,10 +1126,10 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     const Window wn = load_window(st);
     const uint32_t lo = wn.lo, hi = wn.hi, shift = wn.shift, that_key = wn.that;
-    const uint32_t k = bucket_k(g, b);
-    const uint64_t bn = bucket_count(g, b);
+    const uint32_t k = bucket_k(g, bk, b);
+    const uint64_t bn = bucket_count(g, bk, b);
     uint32_t r0, r1;
-    block_regions(g, b, s, &r0, &r1);
+    block_regions(g, bk, b, s, &r0, &r1);
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const uint64_t below = (1ull << lane) - 1ull;
@@ -1098,11 +1139,11 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
     const uint32_t wr1 = wr0 + pw < r1 ? wr0 + pw : r1;
     const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
     const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-    float* rp = residual + (uint64_t)b * g.bucket_elems;
+    float* rp = bucket_residual(g, bk, b);
     uint32_t* hw = w.hist_w + (uint64_t)b * kWinBins;
     uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
     uint32_t* above_of = w.blk_above + (uint64_t)b * kNSub;
-    uint32_t* out = (uint32_t*)(wire + (uint64_t)b * wire_stride);
+    uint32_t* out = bucket_wire(g, bk, b);
 
     // ---- slots of the first kTailRegs regions into registers, every load issued at once
     uint32_t ccnt[kTailRegs], cidx[kTailRegs], cbits[kTailRegs];
@@ -1400,7 +1441,7 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(float* residual, Geomet
     // the exact selection for a bucket the window could not finish (S_OK stays 0)
     if (failed) {
         uint32_t T;
-        if (!bucket_exact_group(residual, g, w, b, s, wn, wire, wire_stride, lh, scratch, &sh_x[0], limit_ticks, &T)) {
+        if (!bucket_exact_group(bk, g, w, b, s, wn, lh, scratch, &sh_x[0], limit_ticks, &T)) {
             if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
             return;
         }
@@ -1458,7 +1499,19 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     uint64_t cap = 2 * (uint64_t)g->k_full + 4096;
     if (cap > bucket_elems) cap = bucket_elems;
     g->lcap2 = (uint32_t)cap;
+    g->listed = 0;
     return true;
+}
+
+// The three launches of the single-pass path.
+void launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w, bool warm, hipStream_t st) {
+    // the window comes from the previous call's exact threshold when there was one
+    if (!warm) k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(bk, g, w);
+    const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
+    k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(bk, g, w);
+    // 100 MHz ticks a block may wait at a barrier before it gives up
+    const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
+    k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(bk, g, w, limit);
 }
 
 // Workspaces whose state words hold a window prediction: address -> shape of the last
@@ -1551,13 +1604,12 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     const uint32_t bx_t = clamp_u32(bx < g.tiles ? bx : g.tiles, 1, 65535);
     const bool warm = take_warm(workspace, g, ratio, fast) && tuning().topk_warm != 0;
     if (fast) {
-        // the window comes from the previous call's exact threshold when there was one
-        if (!warm) k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(grad, residual, g, w);
-        const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
-        k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(grad, residual, g, w);
-        // 100 MHz ticks a block may wait at a barrier before it gives up
-        const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
-        k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride, limit);
+        Buckets bk = {};
+        bk.grad = grad;
+        bk.residual = residual;
+        bk.wire = (uint8_t*)wire;
+        bk.wire_stride = wire_stride;
+        launch_single_pass(bk, g, w, warm, st);
     } else {
         const uint64_t zw = zeroed_words(g);
         k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);
@@ -1569,6 +1621,52 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
         k_topk_count<<<dim3(bx_t, g.nbuckets), kBlock, 0, st>>>(residual, g, w, 0);
         k_topk_emit<<<dim3(bx_t, g.nbuckets), kBlock, 0, st>>>(residual, g, w, (uint8_t*)wire, wire_stride, 0);
     }
+    return launch_status();
+}
+
+uint64_t mccl_hip_topk_list_workspace_bytes(const uint64_t* host_counts, uint32_t nbuckets, double ratio) {
+    if (!host_counts || nbuckets == 0 || nbuckets > kMaxListed) return 0;
+    uint64_t longest = 0;
+    for (uint32_t b = 0; b < nbuckets; b++) {
+        if (host_counts[b] == 0) return 0;
+        longest = host_counts[b] > longest ? host_counts[b] : longest;
+    }
+    return mccl_hip_topk_workspace_bytes(longest * nbuckets, longest, ratio);
+}
+
+int mccl_hip_topk_compress_list(const float* const* host_grads, float* const* host_residuals,
+                                const uint64_t* host_counts, void* const* host_wires,
+                                const uint64_t* host_wire_capacities, uint32_t nbuckets, double ratio,
+                                void* workspace, uint64_t workspace_bytes, void* stream) {
+    if (!host_grads || !host_residuals || !host_counts || !host_wires || !host_wire_capacities || !workspace)
+        return MCCL_HIP_ERR_ARG;
+    if (nbuckets == 0 || nbuckets > kMaxListed || !(ratio > 0.0 && ratio <= 1.0)) return MCCL_HIP_ERR_ARG;
+    Buckets bk = {};
+    uint64_t longest = 0;
+    for (uint32_t b = 0; b < nbuckets; b++) {
+        if (!host_grads[b] || !host_residuals[b] || !host_wires[b] || ((uintptr_t)host_wires[b] & 3))
+            return MCCL_HIP_ERR_ARG;
+        if (host_counts[b] == 0 || host_counts[b] > 0xFFFFFFFFull) return MCCL_HIP_ERR_ARG;  // indices are 32-bit
+        const uint32_t k = mccl_hip_topk_k(host_counts[b], ratio);
+        if (host_wire_capacities[b] < 4 + 8 * (uint64_t)k) return MCCL_HIP_ERR_CAPACITY;
+        bk.lgrad[b] = host_grads[b];
+        bk.lresidual[b] = host_residuals[b];
+        bk.lwire[b] = (uint8_t*)host_wires[b];
+        bk.lcount[b] = (uint32_t)host_counts[b];
+        bk.lk[b] = k;
+        longest = host_counts[b] > longest ? host_counts[b] : longest;
+    }
+    Geometry g;
+    if (!make_geometry(longest * nbuckets, longest, ratio, &g)) return MCCL_HIP_ERR_ARG;
+    g.listed = 1;
+    if (workspace_bytes < workspace_words(g) * 4 + 16) return MCCL_HIP_ERR_WORKSPACE;
+    int rc = mccl_hip_init();
+    if (rc) return rc;
+    void* aligned = (void*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
+    Workspace w = carve(aligned, g);
+    // a list changes from call to call: every call samples
+    mccl_hip_topk_workspace_forget(workspace);
+    launch_single_pass(bk, g, w, false, (hipStream_t)stream);
     return launch_status();
 }
 

@@ -146,6 +146,36 @@ def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
     return wire, stride
 
 
+def topk_compress_list(grads: Sequence[torch.Tensor], residuals: Sequence[torch.Tensor], ratio: float,
+                       wires: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None):
+    """Top-k payloads of a list of separate buckets in one call; returns the list of wire tensors
+    (each max_compressed_size bytes, the payload at its front).  residuals are updated."""
+    nb = len(grads)
+    if nb == 0 or nb != len(residuals):
+        raise ValueError("one residual per gradient bucket, at least one bucket")
+    for i, (g, r) in enumerate(zip(grads, residuals)):
+        _dev(g, f"grads[{i}]", torch.float32, 1)
+        _dev(r, f"residuals[{i}]", torch.float32)
+        if r.numel() != g.numel():
+            raise ValueError(f"residuals[{i}] holds {r.numel()} elements, the bucket {g.numel()}")
+    if wires is None:
+        wires = [torch.empty(topk_wire_stride(g.numel(), ratio), dtype=torch.uint8, device=g.device) for g in grads]
+    for i, w in enumerate(wires):
+        _dev(w, f"wires[{i}]", torch.uint8)
+    counts = (C.c_uint64 * nb)(*[g.numel() for g in grads])
+    caps = (C.c_uint64 * nb)(*[w.numel() for w in wires])
+    if workspace is None:
+        nbytes = int(_lib.load().mccl_hip_topk_list_workspace_bytes(counts, nb, ratio))
+        if nbytes == 0:
+            raise _lib.MCCLHipError(-6, "topk_list_workspace_bytes")
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=grads[0].device)
+    _dev(workspace, "workspace", torch.uint8)
+    rc = _lib.load().mccl_hip_topk_compress_list(_ptrs(grads), _ptrs(residuals), counts, _ptrs(wires), caps, nb,
+                                                ratio, workspace.data_ptr(), workspace.numel(), _stream())
+    _lib.check(rc, "topk_compress_list")
+    return list(wires)
+
+
 def topk_workspace_forget(workspace: torch.Tensor) -> None:
     """The next compress call with this workspace samples the gradient afresh."""
     _lib.check(_lib.load().mccl_hip_topk_workspace_forget(workspace.data_ptr()), "topk_workspace_forget")

@@ -216,3 +216,34 @@ def test_two_bucket_residual_isolation(k):
             w, _ = oracle.topk_compress(g, res[bid], 0.1)
             assert wire.cpu().numpy().tobytes() == w.tobytes(), (step, bid)
     assert float(comp.error_feedback_buffer(C._compression_stable_id(bufs[2])).abs().max()) < 1e-2
+
+
+def test_compress_many_equals_per_bucket_calls_and_the_oracle(k):
+    # a coalesced list of buckets of different sizes, error feedback carried over two steps
+    C = k["C"]
+    rng = np.random.default_rng(9)
+    sizes = [655_360] * 6 + [300_001, 65_537, 4_097, 1_000_003, 13]
+    many, single = C.TopKCompressor(0.01), C.TopKCompressor(0.01)
+    res_o = [np.zeros(n, np.float32) for n in sizes]
+    bufs = [torch.empty(n, device=DEV) for n in sizes]
+    for step in range(2):
+        grads = [student_t(rng, n) * np.float32(10.0 ** (i % 3)) for i, n in enumerate(sizes)]
+        for buf, g in zip(bufs, grads):
+            buf.copy_(torch.from_numpy(g))
+        ids = [100 + i for i in range(len(sizes))]
+        payloads = many.compress_many(bufs, stable_ids=ids)
+        torch.cuda.synchronize()
+        for i, (g, p) in enumerate(zip(grads, payloads)):
+            w, rc = oracle.topk_compress(g, res_o[i], 0.01)
+            assert p.numel() == rc and p.cpu().numpy().tobytes() == w.tobytes(), (step, i)
+            assert np.array_equal(bits(many.error_feedback_buffer(ids[i]).cpu().numpy()), bits(res_o[i])), (step, i)
+            one = single.compress(bufs[i], stable_id=ids[i])
+            assert torch.equal(one, p), (step, i)
+    assert many.error_feedback_buffer_count() == len(sizes)
+    # default ids = storage addresses; an id twice in one call is refused
+    assert len(many.compress_many(bufs[:3])) == 3
+    with pytest.raises(RuntimeError, match="same stable id twice"):
+        many.compress_many(bufs[:2], stable_ids=[1, 1])
+    with pytest.raises(RuntimeError, match="float32 only"):
+        many.compress_many([bufs[0].half()])
+    assert many.compress_many([]) == []

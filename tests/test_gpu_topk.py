@@ -371,3 +371,28 @@ def test_tensor_layer_checks_secondary_buffers(ops):
         ops.cast_f32_to_f16(g, torch.empty(10, dtype=torch.float16, device=DEV))
     with pytest.raises(ValueError, match="dst must be torch.float32"):
         ops.cast_f16_to_f32(g.half(), torch.empty(1000, dtype=torch.float16, device=DEV))
+
+
+def test_compress_list_equals_one_call_per_bucket(ops):
+    """Separate bucket buffers of different lengths (one of them misaligned, one with a single
+    element) through the list entry point: the bytes of one call per bucket, two steps."""
+    from mccl_amd._lib import MCCLHipError
+    rng = np.random.default_rng(12)
+    sizes = [655_360, 300_001, 1, 65_537, 4_097, 1_000_003, 13, 262_144]
+    res_o = [(rng.standard_normal(n) * 1e-4).astype(np.float32) for n in sizes]
+    dres = [to_dev(r, F32, i % 2) for i, r in enumerate(res_o)]
+    for step in range(2):
+        grads = [student_t(rng, n) * np.float32(10.0 ** (i % 4 - 2)) for i, n in enumerate(sizes)]
+        dg = [to_dev(g, F32, (i + 1) % 3) for i, g in enumerate(grads)]
+        wires = ops.topk_compress_list(dg, dres, 0.01)
+        for i, (g, w) in enumerate(zip(grads, wires)):
+            ww, rc = oracle.topk_compress(g, res_o[i], 0.01)
+            assert w.cpu().numpy()[:rc].tobytes() == ww.tobytes(), (step, i)
+            assert np.array_equal(bits(to_np(dres[i], F32)), bits(res_o[i])), (step, i)
+            assert np.array_equal(to_np(dg[i], F32), g)
+    with pytest.raises(MCCLHipError, match="buffer too small"):
+        ops.topk_compress_list(dg[:2], dres[:2], 0.01, wires=[wires[0], torch.empty(8, dtype=torch.uint8, device=DEV)])
+    with pytest.raises(MCCLHipError):
+        ops.topk_compress_list([dg[0]] * 65, [dres[0]] * 65, 0.01)
+    with pytest.raises(ValueError, match="residuals\\[1\\] holds"):
+        ops.topk_compress_list(dg[:2], [dres[0], dres[0]], 0.01)
