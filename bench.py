@@ -51,6 +51,13 @@ def main() -> int:
     import numpy as np
     import torch
     from mccl_amd import hip_ops as ops
+    from mccl_amd import hbm_traffic
+
+    # HBM bytes per launch from the committed counter runs; None (with the reason) when they were
+    # taken on other versions of the kernel sources or another workload size
+    traffic, traffic_note = hbm_traffic.load_for_bench()
+    if a.elems != N_GRAD:
+        traffic, traffic_note = None, "counter runs exist for the default workload size only"
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -102,15 +109,23 @@ def main() -> int:
         "bound": "hbm", "kernel": "k_ring_fold<f32,add>",
         "achieved": rate(fold_bytes, st["avg_ms"]), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": rate(fold_bytes, st["avg_ms"]) / HBM_PEAK_GBPS,
-        # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded in
-        # profiles/ring_fold_f32_w8_96M_hbm_traffic.md (valid for the default workload only)
-        "traffic": 3_478_715_600 if N == N_GRAD else None,
+        "traffic": traffic["ring_fold_f32_w8"] if traffic else None, "traffic_source": traffic_note,
         "bytes_per_launch": fold_bytes, "avg_launch_ms": st["avg_ms"], "min_launch_ms": st["min_ms"],
     }
 
     # device-to-device copy ceiling with the same timing method (read N, write N)
     cpy_ms = stats(gpu_time(lambda: out.copy_(ranks[0]))[1])
     extra["d2d_copy_GBps"] = rate(8 * N, cpy_ms["avg_ms"])
+
+    if a.only in ("all", "fold"):
+        # world sizes the kernel has no compile-time instance for (the reference's tests use 3 and 6)
+        for ws_rt in (3, 6):
+            inv = float(np.float32(1.0 / ws_rt))
+            r = stats(gpu_time(lambda: ops.ring_fold(out, ranks[:ws_rt], ops.AVG, ops.RING_BASIC,
+                                                     bucket_elems=BUCKET, scale_by=inv))[1])
+            b = (ws_rt + 1) * 4 * N
+            extra[f"ring_fold_f32_w{ws_rt}"] = {"ms": r["avg_ms"], "GBps": rate(b, r["avg_ms"]),
+                                                "frac": rate(b, r["avg_ms"]) / HBM_PEAK_GBPS}
 
     if a.only == "all":
         # ---- step-wise drop-in sequence: 7 binary folds per chunk view + scale --
@@ -199,13 +214,13 @@ def main() -> int:
                                           "bytes": topk_bytes, "buckets": nb, "k_per_bucket": ks[0],
                                           "single_pass_buckets": ops.topk_path_report(wsb, N, BUCKET, 0.01)[0]}
         # second half of the headline metric: same fields as `roofline`, for the whole
-        # compress call (six launches); traffic from the FETCH_SIZE / WRITE_SIZE counter
-        # runs in profiles/topk_and_sparse_accumulate_hbm_traffic.md (default workload only)
-        roofline_topk = {"bound": "hbm", "kernel": "mccl_hip_topk_compress (6 launches, dominant k_topk_pass_a_fast)",
+        # compress call (three launches: sample, streaming pass, selection)
+        roofline_topk = {"bound": "hbm", "kernel": "mccl_hip_topk_compress (3 launches, dominant k_topk_pass_a_fast)",
                          "achieved": rate(topk_bytes, tk["avg_ms"]), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": rate(topk_bytes, tk["avg_ms"]) / HBM_PEAK_GBPS,
-                         "traffic": 1_236_252_262 if N == N_GRAD else None,
-                         "bytes_per_launch": topk_bytes, "avg_launch_ms": tk["avg_ms"], "min_launch_ms": tk["min_ms"]}
+                         "traffic": traffic["topk_compress"] if traffic else None, "traffic_source": traffic_note,
+                         "bytes_per_launch": topk_bytes, "avg_launch_ms": tk["avg_ms"],
+                         "median_launch_ms": tk["median_ms"], "min_launch_ms": tk["min_ms"]}
         # one bucket alone (the reference's call granularity; cache resident)
         r1 = residual0[:BUCKET].clone()
         ws1 = ops.topk_workspace(BUCKET, BUCKET, 0.01, dev)
@@ -213,7 +228,26 @@ def main() -> int:
         tb = stats(gpu_time(lambda: ops.topk_compress(grad[:BUCKET], r1, 0.01, wire=w1, workspace=ws1,
                                                       wire_stride=stride))[1])
         extra["config4_topk_one_bucket"] = {"ms": tb["avg_ms"],
-                                            "GBps": rate(12 * BUCKET + 8 * ks[0] + 4, tb["avg_ms"])}
+                                            "GBps": rate(12 * BUCKET + 8 * ks[0] + 4, tb["avg_ms"]),
+                                            "frac": rate(12 * BUCKET + 8 * ks[0] + 4, tb["avg_ms"]) / HBM_PEAK_GBPS}
+        # the reference compresses bucket by bucket (TopKCompressor::compress per DDP bucket): the 15
+        # buckets as 15 separate buffers, through 15 calls and through one list call
+        import torch.distributed  # noqa: F401
+        from mccl_amd import _C
+        bufs = [grad[b * BUCKET: min(N, (b + 1) * BUCKET)] for b in range(nb)]
+        ids = list(range(1, nb + 1))
+        comp = _C.TopKCompressor(0.01)
+        per = stats(gpu_time(lambda: [comp.compress(t, stable_id=i) for t, i in zip(bufs, ids)],
+                             steps=max(3, K // 2))[1])
+        extra["config4_15_compress_calls"] = {"ms": per["avg_ms"], "GBps": rate(topk_bytes, per["avg_ms"]),
+                                              "frac": rate(topk_bytes, per["avg_ms"]) / HBM_PEAK_GBPS,
+                                              "note": "15 x TopKCompressor::compress, 45 launches: bound by the host's launch rate"}
+        comp = _C.TopKCompressor(0.01)
+        many = stats(gpu_time(lambda: comp.compress_many(bufs, stable_ids=ids))[1])
+        extra["config4_compress_many"] = {"ms": many["avg_ms"], "GBps": rate(topk_bytes, many["avg_ms"]),
+                                          "frac": rate(topk_bytes, many["avg_ms"]) / HBM_PEAK_GBPS,
+                                          "note": "TopKCompressor::compress_many on the same 15 buffers: 3 launches"}
+        del comp, bufs
 
         # ---- config 5: decompress-accumulate of 8 ranks' payloads -----------------
         shared = torch.rand(N, generator=gens[4], device=dev) < 0.004
@@ -234,7 +268,9 @@ def main() -> int:
                                                           scale_by=0.125, status=status, workspace=sws))[1])
         extra["config5_sparse_accumulate"] = {"ms": sa["avg_ms"], "GBps": rate(acc_bytes, sa["avg_ms"]),
                                               "frac": rate(acc_bytes, sa["avg_ms"]) / HBM_PEAK_GBPS,
-                                              "bytes": acc_bytes, "status": int(status)}
+                                              "bytes": acc_bytes, "status": int(status),
+                                              "traffic": traffic["sparse_accumulate"] if traffic else None,
+                                              "traffic_source": traffic_note}
 
     if a.only == "all":
         # ---- FP16 compressor casts over the whole gradient (6 B / element each way) ----
@@ -254,33 +290,38 @@ def main() -> int:
         nbk = min(2, (N + BUCKET - 1) // BUCKET)     # bounded sample: 2 buckets of the 15
         cn = min(N, nbk * BUCKET)
         host = [r[:cn].cpu().numpy() for r in ranks]
-        t0 = time.perf_counter()
-        reps = 0
+        # The reference folds in place: a rank's chunk is `local`, the partial that arrived is
+        # `incoming`, and local (op)= incoming (csrc/backend/ProcessGroupMCCL.cpp:492-512).  The
+        # simulated ranks' buffers are therefore folded where they lie - no allocation or copy in
+        # the timed loop - and only throughput is read off (the values drift from pass to pass).
+        times = []
+        t_all = time.perf_counter()
         while True:
+            t0 = time.perf_counter()
             for b in range(nbk):
                 lo, hi = b * BUCKET, min(cn, (b + 1) * BUCKET)
                 ce = (hi - lo + W - 1) // W
-                acc_np = np.empty(hi - lo, np.float32)
                 for c in range(W):
                     s, e = lo + c * ce, min(hi, lo + (c + 1) * ce)
                     if s >= e:
                         continue
-                    part = host[c][s:e].copy()
+                    part = host[c][s:e]
                     for j in range(1, W):
-                        local = host[(c + j) % W][s:e].copy()
+                        local = host[(c + j) % W][s:e]
                         oracle.fold2(local, part, oracle.F32, oracle.OP_SUM, threads=0)  # reference job split
                         part = local
-                    acc_np[s - lo:e - lo] = part
-                oracle.scale(acc_np, oracle.F32, 0.125, threads=0)
-            reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 8:
+                    oracle.scale(part, oracle.F32, 0.125, threads=0)
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - t_all > 10.0 or len(times) >= 12:
                 break
-        cpu_s = (time.perf_counter() - t0) / reps
-        cpu = {"value": (W + 1) * 4 * cn / cpu_s / 1e9, "unit": "GB/s", "cores": min(8, os.cpu_count() or 1),
-               "kind": "port",
+        reps = len(times)
+        cpu_s = sum(times) / reps
+        cpu_med = sorted(times)[reps // 2]
+        cpu = {"value": (W + 1) * 4 * cn / cpu_s / 1e9, "median": (W + 1) * 4 * cn / cpu_med / 1e9,
+               "unit": "GB/s", "cores": min(8, os.cpu_count() or 1), "kind": "port",
                "sample": f"{nbk} of {(N + BUCKET - 1) // BUCKET} buckets ({cn} elements), {reps} repetitions; "
-                         "step-wise ring folds with the reference's job split (>= 1 Mi floats per job, <= 8 jobs), "
-                         "same 36 B/element numerator",
+                         "step-wise ring folds in place with the reference's job split (>= 1 Mi floats per job, "
+                         "<= 8 jobs), timed loop = folds and scale only, same 36 B/element numerator",
                "host_cores_visible": os.cpu_count()}
         if a.only in ("all", "topk") and oracle.RefCompressor.available():
             ref = oracle.RefCompressor(2, 0.01)
@@ -313,7 +354,7 @@ def main() -> int:
         "metric": "HBM GB/s (% of peak) for fp32 bucket fold and top-k 1% compress, 1 GPU",
         "value": fold_gbps, "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": WU,
         "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic (seeded device generators; values as the configs specify)",
         "config": {"workload": "configs[1]: fp32 ring reduce-scatter fold, 8 simulated ranks in one GPU's HBM, "
                                f"{N}-element gradient, 25 MiB buckets x 8 chunks, 7 folds per chunk slot in "
                                "ring-step order, AVG x 1/8 fused",

@@ -1,0 +1,116 @@
+"""Turns two ``rocprofv3 --pmc`` runs of ``bench.py`` (FETCH_SIZE, then WRITE_SIZE)
+into ``profiles/hbm_traffic.json``: HBM bytes per launch of the fold, the top-k
+compress call and the sparse accumulate call, each counter scaled by what the
+same counter reads for a device-to-device copy of known size in the same run.
+
+    python -m mccl_amd.hbm_traffic <fetch_counter_collection.csv> <write_counter_collection.csv>
+
+``bench.py`` reads the JSON for its ``roofline.traffic`` fields and only trusts it
+while the kernel sources it was measured on are unchanged (their SHA-256 is
+stored in the file).
+"""
+from __future__ import annotations
+
+import csv
+import hashlib
+import json
+import os
+import sys
+from collections import defaultdict
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+OUT = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+SOURCES = ["common.hip.h", "fold.hip", "topk.hip", "sparse.hip"]
+N_GRAD = 96_510_024
+COPY_KIB = N_GRAD * 4 / 1024.0          # bench.py's torch copy_ of one rank buffer
+
+
+def source_hashes() -> dict:
+    out = {}
+    for name in SOURCES:
+        with open(os.path.join(HERE, "csrc", name), "rb") as f:
+            out[name] = hashlib.sha256(f.read()).hexdigest()
+    return out
+
+
+def per_kernel(path: str, counter: str) -> dict:
+    """kernel short name -> list of counter values (one per dispatch), whole-gradient launches only."""
+    vals = defaultdict(list)
+    with open(path, newline="") as f:
+        for row in csv.DictReader(f):
+            if row["Counter_Name"] != counter:
+                continue
+            name = row["Kernel_Name"]
+            for key in ("k_ring_fold", "k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail", "k_sparse_bounds",
+                        "k_sparse_accumulate", "copyBuffer"):
+                if key in name:
+                    vals[key].append((int(row["Grid_Size"]), float(row["Counter_Value"])))
+                    break
+    out = {}
+    for key, lst in vals.items():
+        if key == "copyBuffer":
+            # the copy kernel's grid does not depend on the size: the whole-buffer copies are
+            # the ones with the largest counter values
+            top = max(v for _, v in lst)
+            sel = [v for _, v in lst if v > 0.98 * top]
+        else:
+            top = max(g for g, _ in lst)                  # the whole-gradient launches have the largest grid
+            sel = [v for g, v in lst if g == top]
+        out[key] = sum(sel) / len(sel)
+    return out
+
+
+def main(argv) -> int:
+    if len(argv) != 3:
+        print(__doc__)
+        return 2
+    fetch = per_kernel(argv[1], "FETCH_SIZE")
+    write = per_kernel(argv[2], "WRITE_SIZE")
+    # counter units: KiB per dispatch after calibration on the copy of known size
+    f_fac = COPY_KIB / fetch["copyBuffer"]
+    w_fac = COPY_KIB / write["copyBuffer"]
+    kernels = {}
+    for k in sorted(set(fetch) | set(write)):
+        if k == "copyBuffer":
+            continue
+        kernels[k] = {"read_bytes": round(fetch.get(k, 0.0) * f_fac * 1024),
+                      "written_bytes": round(write.get(k, 0.0) * w_fac * 1024)}
+
+    def total(names):
+        return sum(kernels[n]["read_bytes"] + kernels[n]["written_bytes"] for n in names if n in kernels)
+
+    doc = {
+        "what": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, 96,510,024-element workloads of bench.py",
+        "calibration": {"copy_bytes": N_GRAD * 4, "fetch_factor": f_fac, "write_factor": w_fac},
+        "sources_sha256": source_hashes(),
+        "kernels": kernels,
+        "calls": {
+            "ring_fold_f32_w8": total(["k_ring_fold"]),
+            "topk_compress": total(["k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail"]),
+            "sparse_accumulate": total(["k_sparse_bounds", "k_sparse_accumulate"]),
+        },
+    }
+    os.makedirs(os.path.dirname(OUT), exist_ok=True)
+    with open(OUT, "w") as f:
+        json.dump(doc, f, indent=1)
+        f.write("\n")
+    print(json.dumps(doc["calls"]))
+    return 0
+
+
+def load_for_bench():
+    """(calls dict or None, note).  None when the file is missing or was measured on other kernel sources."""
+    try:
+        with open(OUT) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        return None, "profiles/hbm_traffic.json missing"
+    stale = [n for n, h in source_hashes().items() if doc.get("sources_sha256", {}).get(n) != h]
+    if stale:
+        return None, "profiles/hbm_traffic.json was measured on other versions of " + ", ".join(stale)
+    return doc["calls"], "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, same kernel sources)"
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv))
