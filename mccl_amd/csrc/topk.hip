@@ -704,9 +704,11 @@ __device__ __forceinline__ void block_regions(const Geometry& g, BucketsArg bk, 
 // Nothing else happens here: returning atomics and histogram flushes in these
 // 12,000 streaming blocks each cost 7-15 % of the kernel's time when they were
 // tried.
-__global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(Buckets, Geometry g, Workspace w) {
+constexpr int kAWaves = kATile / kRegion;  // wavefronts (= regions) per streaming block; 1, 2 and 8 measured the same or worse
+constexpr int kAThreads = kAWaves * kWave;
+__global__ __launch_bounds__(kAThreads) void k_topk_pass_a_fast(Buckets, Geometry g, Workspace w) {
     const BucketsArg bk = buckets_arg();
-    __shared__ uint32_t stage[kBlock / kWave][kRegSlots][2];
+    __shared__ uint32_t stage[kAWaves][kRegSlots][2];
     const uint32_t b = blockIdx.y, t = blockIdx.x;
     const uint64_t bn = bucket_count(g, bk, b);
     const int lane = threadIdx.x & (kWave - 1);
@@ -714,14 +716,13 @@ __global__ __launch_bounds__(kBlock) void k_topk_pass_a_fast(Buckets, Geometry g
     const uint64_t w0 = (uint64_t)t * kATile + (uint64_t)wave * kRegion;  // first element of this wave's region
     if (t == 0) {
         // the words the selection kernel accumulates into start every call at zero
-        static_assert(kWinBins == kBlock, "one histogram bin per thread");
-        w.hist_w[(uint64_t)b * kWinBins + threadIdx.x] = 0;
+        for (int i = threadIdx.x; i < kWinBins; i += kAThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
         if (threadIdx.x == 0) {
             uint32_t* st = w.state + (uint64_t)b * kStateWords;
             st[S_BAR1] = 0; st[S_BAR2] = 0; st[S_N2] = 0; st[S_OK] = 0; st[S_TIMEOUT] = 0;
             st[S_BARF] = 0; st[S_BARF + 1] = 0; st[S_BARF + 2] = 0; st[S_BARF + 3] = 0;
         }
-        for (int i = threadIdx.x; i < kHistWords; i += kBlock) w.hist[(uint64_t)b * kHistWords + i] = 0;
+        for (int i = threadIdx.x; i < kHistWords; i += kAThreads) w.hist[(uint64_t)b * kHistWords + i] = 0;
     }
     if (w0 >= bn) return;  // whole wavefront; the kernel has no barriers
     const float* gp = bucket_grad(g, bk, b) + w0;
@@ -1284,18 +1285,21 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Wo
     }
 
     // ---- phase 3: exact threshold from list2 (every block, redundantly) -----------------
-    const uint32_t count2 = ld_agent(st + S_N2);
-    if (count2 > g.lcap2) {  // more keys in the threshold bin than list2 holds (heavy ties)
-        failed = true;
-        break;
-    }
+    // every load of this phase is issued at once: the entries do not wait for their count
+    // (slots past it hold leftovers and are masked below)
     constexpr int kL2Regs = 4;  // list2 entries per thread kept in registers (1024 per block)
     uint32_t eidx[kL2Regs], ekey[kL2Regs];
 #pragma unroll
     for (int j = 0; j < kL2Regs; j++) {
         const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
-        eidx[j] = i < count2 ? ld_agent(&l2[2 * (uint64_t)i]) : 0u;
-        ekey[j] = i < count2 ? ld_agent(&l2[2 * (uint64_t)i + 1]) : 0u;
+        eidx[j] = i < g.lcap2 ? ld_agent(&l2[2 * (uint64_t)i]) : 0u;
+        ekey[j] = i < g.lcap2 ? ld_agent(&l2[2 * (uint64_t)i + 1]) : 0u;
+    }
+    const uint32_t above_mine = threadIdx.x < (uint32_t)kNSub ? ld_agent(&above_of[threadIdx.x]) : 0u;
+    const uint32_t count2 = ld_agent(st + S_N2);
+    if (count2 > g.lcap2) {  // more keys in the threshold bin than list2 holds (heavy ties)
+        failed = true;
+        break;
     }
     auto for_list2 = [&](auto&& body) {
 #pragma unroll
@@ -1347,11 +1351,8 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Wo
     uint32_t l2_before, l2_total, above_before, above_total;
     block_exclusive_scan(mine_before, scratch, &l2_before);
     block_exclusive_scan(mine_all, scratch, &l2_total);
-    {
-        const uint32_t v = threadIdx.x < (uint32_t)kNSub ? ld_agent(&above_of[threadIdx.x]) : 0u;
-        block_exclusive_scan(threadIdx.x < s ? v : 0u, scratch, &above_before);
-        block_exclusive_scan(v, scratch, &above_total);
-    }
+    block_exclusive_scan(threadIdx.x < s ? above_mine : 0u, scratch, &above_before);
+    block_exclusive_scan(above_mine, scratch, &above_total);
     if (above_total + l2_total != k) {  // cannot happen with consistent lists
         failed = true;
         break;
@@ -1508,7 +1509,7 @@ void launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w
     // the window comes from the previous call's exact threshold when there was one
     if (!warm) k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(bk, g, w);
     const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
-    k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kBlock, 0, st>>>(bk, g, w);
+    k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kAThreads, 0, st>>>(bk, g, w);
     // 100 MHz ticks a block may wait at a barrier before it gives up
     const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
     k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(bk, g, w, limit);
@@ -1669,6 +1670,7 @@ int mccl_hip_topk_compress_list(const float* const* host_grads, float* const* ho
     launch_single_pass(bk, g, w, false, (hipStream_t)stream);
     return launch_status();
 }
+
 
 int mccl_hip_topk_path_report(const void* workspace, uint64_t n_total, uint64_t bucket_elems, double ratio,
                               uint32_t* host_single_pass_buckets, uint32_t* host_buckets, void* stream) {
