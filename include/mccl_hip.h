@@ -215,15 +215,19 @@ int mccl_hip_topk_decompress(const void* wire, uint64_t wire_bytes, float* dense
  * host_wires[r] is rank r's payload buffer laid out like the output of
  * mccl_hip_topk_compress (bucket b at + b * wire_stride, indices relative to
  * the bucket).  Every element of acc is written exactly once.  Each payload's
- * k is read on the device; 4 + 8k > wire_stride or an index outside its bucket
- * sets *status (as above) and the offending pairs are skipped.  Pairs within
- * one payload must have ascending indices (what compress emits). */
+ * k is read on the device; 4 + 8k > wire_stride sets *status to
+ * MCCL_HIP_ERR_SIZE (the payload counts as empty), an index outside its bucket
+ * sets MCCL_HIP_ERR_INDEX (the pair is skipped).  Pairs within one payload
+ * must have strictly ascending indices (what compress emits): a payload that
+ * does not sets MCCL_HIP_ERR_INDEX and leaves unspecified values in its
+ * bucket of acc; nothing outside acc is ever written. */
 int mccl_hip_sparse_accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems,
                                const void* const* host_wires, int ws, uint64_t wire_stride,
                                int apply_scale, float scale, int* status, void* workspace,
                                uint64_t workspace_bytes, void* stream);
-/* Scratch for mccl_hip_sparse_accumulate (per rank and bucket, the position in
- * the payload at which every 8192-element output tile begins).  Passing
+/* Scratch for mccl_hip_sparse_accumulate: per rank and bucket, a table of
+ * positions in the payload (where the pairs of each run of output tiles
+ * begin; one entry per 2048 output elements at most).  Passing
  * workspace = NULL is allowed: the ranges are then found by binary search in
  * every block, which costs about 3x the time on MI355X. */
 uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, int ws);
@@ -231,7 +235,7 @@ uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t b
 /* mccl_hip_sparse_accumulate for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc).  No counterpart in the reference.  Same arguments, meaning and
- * results as mccl_hip_sparse_accumulate with a workspace, but the tile-bounds
+ * results as mccl_hip_sparse_accumulate with a workspace, but the position
  * table lives in a MCCL_HIP_SPARSE_STATIC_BYTES array inside the library's
  * device image (one copy per GPU, held until the process ends), and the call
  * itself allocates nothing.  Shapes whose table
@@ -278,7 +282,8 @@ int mccl_hip_fence_block_stream(uint64_t ticket, void* stream);
 int mccl_hip_sync(void* stream);
 
 /* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
-/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_warm", "topk_barrier_ms" */
+/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_warm", "topk_barrier_ms",
+ * "sparse_path" (0 auto, 1 tile kernels only), "sparse_run_steps" (0 auto) */
 int mccl_hip_set_tuning(const char* key, int value);
 int mccl_hip_get_tuning(const char* key);
 

@@ -7,13 +7,19 @@
 //
 // sparse accumulate: the reference decompresses every peer's payload into a
 // dense buffer and folds the dense buffers in ascending rank order
-// (csrc/backend/ProcessGroupMCCL.cpp:1692-1709,:2272-2296).  Here each block
-// owns one 8192-element tile of the output, keeps it in LDS starting at +0.0,
-// and for rank 0, 1, ... adds that rank's pairs that fall inside the tile
-// (found by binary search in the sorted payload; indices are unique within a
-// rank, so a rank's adds never collide), then writes the tile once, scaled.
-// HBM traffic is the algorithmic minimum: every payload read once, every output
-// element written once.
+// (csrc/backend/ProcessGroupMCCL.cpp:1692-1709,:2272-2296).  Here the output is
+// cut into tiles that live in LDS, start at +0.0, receive rank 0's, rank 1's, ...
+// pairs that fall inside them, and are written once, scaled.  Two kernel
+// families do that:
+//   runs of tiles (up to 8 ranks, payloads of the usual density, a workspace):
+//     one wavefront per run of 2048-element tiles, every rank's pairs held in
+//     registers, rank order kept by the LDS's in-order execution of one
+//     wavefront's adds; a small table says in which 64-pair window of each
+//     payload a run begins.
+//   tile kernels (everything else): one block per 8192-element tile with a
+//     barrier between ranks, ranges from a bounds table or by binary search.
+// HBM traffic is close to the algorithmic minimum: every payload read once (plus
+// one index in 64 for the table), every output element written once.
 #include "common.hip.h"
 #include "runtime.h"
 
@@ -58,7 +64,7 @@ struct WirePtrs {
     const uint8_t* w[MCCL_HIP_MAX_WORLD];
 };
 
-// Scratch of mccl_hip_sparse_accumulate_static: the tile-bounds table lives in
+// Scratch of mccl_hip_sparse_accumulate_static: the position table lives in
 // this file-scope device array instead of a caller workspace, so the call
 // allocates nothing.  Every GPU holds its own copy at its own address; host
 // code only ever uses the address hipGetSymbolAddress returned for the device
@@ -297,6 +303,292 @@ __global__ __launch_bounds__(kAccThreads) void k_sparse_accumulate_b(float* acc,
     }
 }
 
+// ---- runs of tiles, one wavefront each ------------------------------------------
+// The kernels above pay for finding where a tile's pairs begin: a table that a
+// pre-pass builds from a second read of every payload.  Here a wavefront owns a
+// run of consecutive 2048-element tiles of one bucket and walks every rank's
+// payload forward as it goes, so a position has to be found only where a run
+// begins, and only to the nearest 64 pairs: the wavefront keeps, for each rank,
+// a window of 64 consecutive pairs in registers (one per lane) plus the next
+// window, already requested.  A pair belongs to the current tile exactly when
+// its index lies inside it; pairs of earlier tiles are behind, pairs of later
+// tiles wait in the window.  When a window's last index is below the tile's end
+// the next window is swapped in and looked at for the same tile.  The tile sits
+// in LDS (8 KiB per wavefront), ranks add in ascending order (the LDS executes
+// one wavefront's operations in order, so no barrier is involved), and the tile
+// goes out once, scaled, in 16-byte stores.  Payload bytes are read once, plus
+// one window where two runs meet.
+//
+// Where a run begins: k_sparse_starts reads one index per 64 pairs (an eighth of
+// the payload's cache lines) and writes, for every run w, the window that holds
+// the last sampled index below the run's first element; every pair before that
+// window belongs to an earlier run.
+constexpr int kRunL = 2048;    // elements per tile of a wavefront
+constexpr int kRunWaves = 4;   // wavefronts (= runs) per block
+constexpr int kRunRanks = 8;   // ranks a wavefront holds windows for; larger worlds use the tile kernels
+constexpr int kWin = kWave;    // pairs per window
+constexpr int kRunWins = 3;    // windows of a rank a wavefront requests when its run begins
+constexpr int kXcds = 8;       // accelerator dies of an MI355X; block B runs on die B mod 8
+
+constexpr int kStartThreads = 1024;
+constexpr uint32_t kStartSamples = 8192;  // samples of one payload the block keeps in LDS (32 KiB)
+
+// One block per (bucket, rank).  The samples (every 64th index) are requested before k is known
+// (inside the payload's capacity, masked afterwards), so the kernel is one round trip: samples
+// into LDS, then every run finds by binary search how many samples lie below its first element.
+__global__ __launch_bounds__(kStartThreads) void k_sparse_starts(WirePtrs wires, int ws, uint64_t wire_stride,
+                                                                 uint32_t run_elems, uint32_t runs, uint32_t* start,
+                                                                 int* status) {
+    __shared__ uint32_t samp[kStartSamples];
+    const uint32_t b = blockIdx.x / (uint32_t)ws, r = blockIdx.x % (uint32_t)ws;
+    const uint32_t* wp = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride);
+    const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
+    const uint32_t cap = (kmax + kWin - 1) / kWin;  // samples the payload can hold (at most kStartSamples)
+    constexpr int kPer = kStartSamples / kStartThreads;
+    uint32_t v[kPer];
+#pragma unroll
+    for (int i = 0; i < kPer; i++) {
+        const uint32_t j = (uint32_t)i * kStartThreads + threadIdx.x;
+        v[i] = j < cap ? wp[1 + 2 * (uint64_t)kWin * j] : 0u;
+    }
+    uint32_t k = wp[0];
+    if (k > kmax) {
+        if (status) *status = MCCL_HIP_ERR_SIZE;
+        k = 0;
+    }
+    const uint32_t nsamp = (k + kWin - 1) / kWin;
+#pragma unroll
+    for (int i = 0; i < kPer; i++) {
+        const uint32_t j = (uint32_t)i * kStartThreads + threadIdx.x;
+        if (j < cap) samp[j] = v[i];
+    }
+    __syncthreads();
+    uint32_t* st = start + ((uint64_t)b * ws + r) * runs;
+    for (uint32_t w = threadIdx.x; w < runs; w += kStartThreads) {
+        // samples below the run's first element; the last of them names the window to begin in.
+        // (Unsorted samples give some window or other; the accumulate kernel trusts no entry.)
+        const uint64_t first = (uint64_t)w * run_elems;
+        uint32_t lo = 0, hi = nsamp;
+        while (lo < hi) {
+            const uint32_t mid = lo + ((hi - lo) >> 1);
+            if (samp[mid] < first) lo = mid + 1;
+            else hi = mid;
+        }
+        st[w] = lo ? (lo - 1) * kWin : 0u;
+    }
+}
+
+typedef const __attribute__((address_space(1))) uint32_t* GlobalWords;  // loads compile to global_load, not flat_load
+
+// One window of a rank's pairs: lane l asks for pair base + l.  The load is unconditional (no
+// branch, so the loads of all ranks and windows are in flight together): positions past the
+// payload's capacity are clamped to its last pair (kmax >= 1) and sorted out by window_index.
+__device__ __forceinline__ u2a4 load_window(GlobalWords pairs, uint32_t base, uint32_t kmax, int lane) {
+    uint32_t pos = base + (uint32_t)lane;
+    if (pos > kmax - 1) pos = kmax - 1;
+    return *(const __attribute__((address_space(1))) u2a4*)(pairs + 2 * (uint64_t)pos);
+}
+
+// The index a lane holds: lanes at or past k hold 0xFFFFFFFF, which lies in no tile.
+__device__ __forceinline__ uint32_t window_index(u2a4 v, uint32_t base, uint32_t k, int lane) {
+    return base + (uint32_t)lane < k ? v[0] : 0xFFFFFFFFu;
+}
+
+// Indices of a window ascend, continue the pair before the window (`before`), and stay inside the bucket.
+// The value the lane below holds (lane 0: `first`): one DPP move, no LDS traffic.
+__device__ __forceinline__ uint32_t from_lane_below(uint32_t v, uint32_t first) {
+    // wave_shr:1 - lane l reads lane l - 1 across the whole wavefront; lane 0 keeps `first`
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138, 0xf, 0xf, false);
+}
+
+// Lanes (as a mask) whose pair breaks the rule: indices of a window ascend, continue the pair
+// before the window (`before`), and stay inside the bucket.  `idx` is what was loaded, before
+// the lanes past k are marked.
+__device__ __forceinline__ uint64_t bad_lanes(uint32_t idx, uint32_t base, uint32_t k, uint32_t before, uint32_t bn) {
+    const uint32_t up = from_lane_below(idx, before);
+    uint64_t m = __ballot(up >= idx);
+    if (base == 0) m &= ~1ull;  // the payload's first pair follows nothing
+    m |= __ballot(idx >= bn);
+    const uint32_t live = k > base ? k - base : 0u;  // lanes that hold a pair of the payload
+    return live >= (uint32_t)kWin ? m : m & ((1ull << live) - 1);
+}
+
+// tile[off] += v as one LDS instruction that returns nothing.  The LDS adds in IEEE single
+// precision, round to nearest even, subnormals kept, and executes one wavefront's instructions in
+// the order they were issued, so successive ranks' adds to one element happen in rank order
+// with no wait between them.
+__device__ __forceinline__ void lds_add(float* p, float v) {
+    (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+}
+
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, int l) {
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, l);
+}
+
+
+// NR: ranks the code is unrolled for (ws <= NR; the ranks past ws read rank 0's payload as if
+// its k were 0).  wire_stride holds at least one pair.
+template <int NR>
+__global__ __launch_bounds__(kRunWaves * kWave, 4) void k_sparse_accumulate_runs(
+    float* acc, uint64_t n_total, uint64_t bucket_elems, WirePtrs wires, int ws, uint64_t wire_stride,
+    uint32_t run_steps, uint32_t runs, uint32_t nbuckets, uint32_t blocks_per_xcd, const uint32_t* start,
+    int apply_scale, float scale, int* status) {
+    __shared__ __attribute__((aligned(16))) float tiles[kRunWaves][kRunL];
+    const int lane = threadIdx.x & (kWave - 1);
+    // the same in every lane; saying so keeps everything derived from it (the run, its tiles,
+    // the window tests) in scalar registers and on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    // blocks go to the XCDs in turn: block B runs on XCD B mod 8.  Each XCD takes one contiguous
+    // eighth of the runs, in order, so the windows that neighbouring runs share are found in
+    // that XCD's L2 and its stores move through memory in one direction.
+    const uint32_t vblock = (blockIdx.x % kXcds) * blocks_per_xcd + blockIdx.x / kXcds;
+    const uint64_t grun = (uint64_t)vblock * kRunWaves + (uint32_t)wave;
+    if (grun >= (uint64_t)runs * nbuckets) return;  // whole wavefront; the kernel has no block barriers
+    const uint32_t b = (uint32_t)(grun / runs), run = (uint32_t)(grun % runs);
+    const uint64_t bstart = (uint64_t)b * bucket_elems;
+    const uint32_t bn = (uint32_t)((n_total - bstart) < bucket_elems ? (n_total - bstart) : bucket_elems);
+    const uint64_t e0 = (uint64_t)run * run_steps * kRunL;
+    if (e0 >= bn) return;
+    const uint64_t e1w = e0 + (uint64_t)run_steps * kRunL;
+    const uint32_t e1 = e1w < bn ? (uint32_t)e1w : bn;  // end of this run
+    const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
+    float* tile = tiles[wave];
+    {
+        const u4a z = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < kRunL / (4 * kWave); i++) ((u4a*)tile)[i * kWave + lane] = z;
+    }
+
+    uint64_t bad = 0;       // lanes that saw a pair out of order or out of range, reported once
+    bool oversize = false;  // a k beyond the payload's capacity
+    // first round trip: every rank's k and the window its pairs of this run begin in
+    uint32_t kk[NR], wnext[NR];
+    GlobalWords pairs[NR];
+    {
+        uint32_t kraw[NR], craw[NR];
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const int rr = r < ws ? r : 0;
+            GlobalWords wp = (GlobalWords)(wires.w[rr] + (uint64_t)b * wire_stride);
+            pairs[r] = wp + 1;
+            kraw[r] = wp[0];
+            craw[r] = ((GlobalWords)start)[((uint64_t)b * ws + rr) * runs + run];
+        }
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            uint32_t k = kraw[r], c = craw[r] & ~(uint32_t)(kWin - 1);
+            if (k > kmax) {
+                oversize = true;
+                k = 0;
+            }
+            if (r >= ws) k = 0;
+            if (c >= k) c = k ? ((k - 1) & ~(uint32_t)(kWin - 1)) : 0u;  // a table entry is never trusted
+            kk[r] = __builtin_amdgcn_readfirstlane(k);
+            wnext[r] = __builtin_amdgcn_readfirstlane(c);
+        }
+    }
+    // second round trip: kRunWins windows of every rank at once; a run of the usual density needs
+    // no other load
+    u2a4 raw[NR][kRunWins];
+    uint32_t before[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        before[r] = pairs[r][2 * (uint64_t)(wnext[r] ? wnext[r] - 1 : 0u)];  // only used when the window is not the first
+#pragma unroll
+        for (int i = 0; i < kRunWins; i++) raw[r][i] = load_window(pairs[r], wnext[r] + (uint32_t)i * kWin, kmax, lane);
+    }
+    // wlast[r][i]: last index of window i, in a scalar register: whether a tile is done with a
+    // window is decided without vector work
+    uint32_t widx[NR][kRunWins], wval[NR][kRunWins], wlast[NR][kRunWins];
+    int nreg[NR];  // windows of the rank still in registers
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        uint32_t prev = lane_value(before[r], 0);
+#pragma unroll
+        for (int i = 0; i < kRunWins; i++) {
+            const uint32_t base = wnext[r] + (uint32_t)i * kWin;
+            bad |= bad_lanes(raw[r][i][0], base, kk[r], prev, bn);
+            widx[r][i] = window_index(raw[r][i], base, kk[r], lane);
+            wval[r][i] = raw[r][i][1];
+            prev = lane_value(widx[r][i], kWin - 1);  // 0xFFFFFFFF once the payload's end is in the window
+            wlast[r][i] = prev;
+        }
+        wnext[r] += kRunWins * kWin;  // the first window not in registers
+        nreg[r] = kRunWins;
+    }
+
+    for (uint32_t ts = (uint32_t)e0; ts < e1; ts += kRunL) {
+        const uint32_t tlen = (e1 - ts) < (uint32_t)kRunL ? (e1 - ts) : (uint32_t)kRunL;
+        const uint32_t tend = ts + tlen;
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            // slot 0 is the window the run has reached; the others wait behind it
+            for (;;) {
+                const uint32_t off = widx[r][0] - ts;
+                if (off < tlen) lds_add(&tile[off], u2f(wval[r][0]));
+                if (wlast[r][0] >= tend) break;  // the rest of the window belongs to later tiles
+                // the window ends inside this tile: the next one may begin in it
+                if (nreg[r] > 1) {
+#pragma unroll
+                    for (int i = 0; i + 1 < kRunWins; i++) {
+                        widx[r][i] = widx[r][i + 1];
+                        wval[r][i] = wval[r][i + 1];
+                        wlast[r][i] = wlast[r][i + 1];
+                    }
+                    nreg[r]--;
+                } else if (wnext[r] < kk[r]) {
+                    // a dense stretch used up the windows requested at the start: further windows
+                    // come one at a time, each waited for
+                    const u2a4 v = load_window(pairs[r], wnext[r], kmax, lane);
+                    bad |= bad_lanes(v[0], wnext[r], kk[r], wlast[r][0], bn);
+                    widx[r][0] = window_index(v, wnext[r], kk[r], lane);
+                    wval[r][0] = v[1];
+                    wlast[r][0] = lane_value(widx[r][0], kWin - 1);
+                    wnext[r] += kWin;
+                } else {
+                    wlast[r][0] = 0xFFFFFFFFu;  // the payload is finished
+                    widx[r][0] = 0xFFFFFFFFu;
+                    break;
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        float* out = acc + bstart + ts;
+        if (tlen == (uint32_t)kRunL && (((uintptr_t)out & 15) == 0)) {
+            // all LDS reads first, so that one wait covers them; then the tile is cleared for the
+            // next round and the stores go out
+            constexpr int kVecs = kRunL / (4 * kWave);
+            u4a v[kVecs];
+#pragma unroll
+            for (int i = 0; i < kVecs; i++) v[i] = ((u4a*)tile)[i * kWave + lane];
+            const u4a z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < kVecs; i++) ((u4a*)tile)[i * kWave + lane] = z;
+            if (apply_scale) {
+#pragma unroll
+                for (int i = 0; i < kVecs; i++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) v[i][q] = f2u(u2f(v[i][q]) * scale);
+            }
+#pragma unroll
+            for (int i = 0; i < kVecs; i++) {
+                __builtin_nontemporal_store(v[i], (u4a*)out + i * kWave + lane);
+            }
+        } else {
+            for (uint32_t i = (uint32_t)lane; i < tlen; i += kWave) {
+                const float x = tile[i];
+                tile[i] = 0.0f;
+                out[i] = apply_scale ? x * scale : x;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (status) {
+        if (bad) *status = MCCL_HIP_ERR_INDEX;
+        if (oversize) *status = MCCL_HIP_ERR_SIZE;
+    }
+}
+
 // Validates the arguments and enqueues the kernels; `workspace` (may be null:
 // scratch-free kernel) is known to be large enough.
 int accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems, const void* const* host_wires, int ws,
@@ -327,6 +619,34 @@ int accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems, const void* 
     }
     uint32_t* start = (uint32_t*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
     const uint64_t kmax = (wire_stride - 4) / 8;
+    // pairs of one rank in a 2048-element tile when the payload is full
+    const uint64_t steps_bucket = (bucket_elems + kRunL - 1) / kRunL;
+    const uint64_t per_tile = (kmax + steps_bucket - 1) / steps_bucket;
+    if (ws <= kRunRanks && tuning().sparse_path != 1 && per_tile <= 96 && kmax >= 1 &&
+        (kmax + kWin - 1) / kWin <= kStartSamples) {
+        // a run is as many tiles as bring about 96 pairs of a rank, half of what the three windows
+        // requested at its start hold: a run of the usual density never loads again
+        uint64_t run_steps = (uint64_t)tuning().sparse_run_steps;
+        if (run_steps == 0) run_steps = per_tile ? 96 / per_tile : 8;
+        if (run_steps > 8 && tuning().sparse_run_steps == 0) run_steps = 8;
+        if (run_steps < 1) run_steps = 1;
+        if (run_steps > steps_bucket) run_steps = steps_bucket;
+        const uint32_t runs = (uint32_t)((steps_bucket + run_steps - 1) / run_steps);
+        k_sparse_starts<<<(uint32_t)(nb * ws), kStartThreads, 0, st>>>(wp, ws, wire_stride,
+                                                                        (uint32_t)(run_steps * kRunL), runs, start, status);
+        const uint64_t blocks = ((uint64_t)runs * nb + kRunWaves - 1) / kRunWaves;
+        const uint32_t per_xcd = (uint32_t)((blocks + kXcds - 1) / kXcds);
+#define MCCLHIP_RUNS(NR)                                                                               \
+    k_sparse_accumulate_runs<NR><<<per_xcd * kXcds, kRunWaves * kWave, 0, st>>>(                        \
+        acc, n_total, bucket_elems, wp, ws, wire_stride, (uint32_t)run_steps, runs, (uint32_t)nb, per_xcd, \
+        start, apply_scale, scale, status)
+        if (ws == 1) MCCLHIP_RUNS(1);
+        else if (ws == 2) MCCLHIP_RUNS(2);
+        else if (ws <= 4) MCCLHIP_RUNS(4);
+        else MCCLHIP_RUNS(8);
+#undef MCCLHIP_RUNS
+        return launch_status();
+    }
     const uint32_t bx = clamp_u32((kmax + kBlock * 8 - 1) / (kBlock * 8), 1, 0x7FFFFFFF);
     k_sparse_bounds<<<dim3(bx, (uint32_t)(nb * ws)), kBlock, 0, st>>>(wp, ws, wire_stride, n_total, bucket_elems,
                                                                         tiles, start, status);
@@ -378,7 +698,8 @@ uint64_t mccl_hip_sparse_accumulate_workspace_bytes(uint64_t n_total, uint64_t b
     if (n_total == 0 || bucket_elems == 0 || ws < 1 || ws > MCCL_HIP_MAX_WORLD) return 0;
     if (bucket_elems > n_total) bucket_elems = n_total;
     const uint64_t nb = (n_total + bucket_elems - 1) / bucket_elems;
-    const uint64_t tiles = (bucket_elems + kAccTile - 1) / kAccTile;
+    // one entry per 2048-element tile: room for the table of either kernel pair
+    const uint64_t tiles = (bucket_elems + kRunL - 1) / kRunL;
     return nb * (uint64_t)ws * (tiles + 1) * 4 + 64;
 }
 

@@ -1,5 +1,5 @@
 """mccl_hip_sparse_accumulate_static (the entry point that allocates nothing: its
-tile-bounds table is a static device array) against mccl_hip_sparse_accumulate
+position table is a static device array) against mccl_hip_sparse_accumulate
 with a caller workspace, bit for bit, through the C ABI: two calls in a row,
 the second on a smaller input, so stale contents of the shared array from the
 first call are in place when the second runs."""
