@@ -293,7 +293,11 @@ __device__ __forceinline__ void pick_bins(const uint32_t* const (&h)[NR], const 
 #pragma unroll
     for (int z = 0; z < NR; z++) {
         uint32_t above = inc[z] - sum[z];
-        for (int w2 = 0; w2 < wave; w2++) above += scratch[z * NW + w2];
+#pragma unroll
+        for (int w2 = 0; w2 < NW; w2++) {  // all reads issued together; a loop up to `wave` waits for each
+            const uint32_t s = scratch[z * NW + w2];
+            if (w2 < wave) above += s;
+        }
 #pragma unroll
         for (int j = 0; j < PER; j++) {
             if (above < remaining[z] && remaining[z] <= above + c[z][j]) {
@@ -571,14 +575,13 @@ __device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32
 }
 
 // One block per bucket.  Loads kSample evenly spread elements of grad + residual
-// into LDS and radix-selects (11 + 10 key bits, all ranks in the same sweeps)
-// the keys of sample ranks
+// (their keys stay in registers, 12 per thread) and radix-selects (11 + 10 key
+// bits, all ranks in the same sweeps) the keys of sample ranks
 //     r_hi = ks - 6 sqrt(ks) - 16,   r_lo = ks + 6 sqrt(ks) + 16   and   ks,
 // ks = k * S / n being the expected number of sampled elements among the top k:
 // the two ends of the candidate window and the predicted threshold.
 __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(Buckets, Geometry g, Workspace w) {
     const BucketsArg bk = buckets_arg();
-    __shared__ uint32_t keys[kSample];
     __shared__ uint32_t lh[3][kBinsR];
     __shared__ uint32_t scratch[3 * (kSampleThreads / kWave + 2)];
     const uint32_t b = blockIdx.x;
@@ -586,24 +589,29 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(Buckets, Geometr
     const float* gp = bucket_grad(g, bk, b);
     const float* rp = bucket_residual(g, bk, b);
     const uint64_t nvec = bn / 4;
-    constexpr int SV = kSample / 4;  // sampled vectors
+    constexpr int SV = kSample / 4;               // sampled vectors
+    constexpr int PV = SV / kSampleThreads;       // vectors per thread; their 4 * PV keys stay in registers
     // sampled in runs of 8 vectors (one 128-byte line per array), runs evenly spread
     const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)(nvec & ~7ull) : (uint32_t)SV;
     const uint64_t stride = nsv ? (nvec / (nsv / 8)) : 8;  // vectors between run starts (>= 8)
-    u4a gv[SV / kSampleThreads], rv[SV / kSampleThreads];
+    u4a gv[PV], rv[PV];
 #pragma unroll
-    for (int j = 0; j < SV / kSampleThreads; j++) {
+    for (int j = 0; j < PV; j++) {
         const uint32_t i = (uint32_t)j * kSampleThreads + threadIdx.x;
         const uint32_t ii = i < nsv ? i : 0;
         const uint64_t v = (uint64_t)(ii >> 3) * stride + (ii & 7);
         gv[j] = nsv ? *(const u4u4*)(gp + v * 4) : u4a{0u, 0u, 0u, 0u};
         rv[j] = nsv ? *(const u4u4*)(rp + v * 4) : u4a{0u, 0u, 0u, 0u};
     }
+    // the histogram is cleared while the loads are under way
+    for (int i = threadIdx.x; i < 3 * kBinsR; i += kSampleThreads) (&lh[0][0])[i] = 0;
+    uint32_t key[PV][4];
+    bool have[PV];
 #pragma unroll
-    for (int j = 0; j < SV / kSampleThreads; j++) {
-        const uint32_t i = (uint32_t)j * kSampleThreads + threadIdx.x;
+    for (int j = 0; j < PV; j++) {
+        have[j] = (uint32_t)j * kSampleThreads + threadIdx.x < nsv;
 #pragma unroll
-        for (int q = 0; q < 4; q++) keys[4 * i + q] = i < nsv ? key_of(u2f(gv[j][q]) + u2f(rv[j][q])) : 0u;
+        for (int q = 0; q < 4; q++) key[j][q] = key_of(u2f(gv[j][q]) + u2f(rv[j][q]));
     }
     const uint32_t S = nsv * 4;
     const float ks = (float)bucket_k(g, bk, b) * (float)S / (float)bn;
@@ -623,16 +631,23 @@ __global__ __launch_bounds__(kSampleThreads) void k_topk_sample(Buckets, Geometr
     for (int r = 0; r < 2; r++) {
         // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves all ranks
         uint32_t* h0 = &lh[0][0];
-        for (int i = threadIdx.x; i < NR * kBinsR; i += kSampleThreads) h0[i] = 0;
-        __syncthreads();
-        for (uint32_t i = threadIdx.x; i < S; i += kSampleThreads) {
-            const uint32_t key = keys[i];
-            if (r == 0) {
-                atomicAdd(&h0[key >> 20], 1u);
-            } else {
+        if (r == 1) {
+            for (int i = threadIdx.x; i < NR * kBinsR; i += kSampleThreads) h0[i] = 0;
+            __syncthreads();
+        }
 #pragma unroll
-                for (int z = 0; z < NR; z++)
-                    if (active[z] && (key >> 20) == (prefix[z] >> 20)) atomicAdd(&lh[z][(key >> 10) & (kBinsR - 1)], 1u);
+        for (int j = 0; j < PV; j++) {
+            if (!have[j]) continue;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t kq = key[j][q];
+                if (r == 0) {
+                    atomicAdd(&h0[kq >> 20], 1u);
+                } else {
+#pragma unroll
+                    for (int z = 0; z < NR; z++)
+                        if (active[z] && (kq >> 20) == (prefix[z] >> 20)) atomicAdd(&lh[z][(kq >> 10) & (kBinsR - 1)], 1u);
+                }
             }
         }
         __syncthreads();
@@ -712,7 +727,7 @@ __global__ __launch_bounds__(kAThreads) void k_topk_pass_a_fast(Buckets, Geometr
     const uint32_t b = blockIdx.y, t = blockIdx.x;
     const uint64_t bn = bucket_count(g, bk, b);
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     const uint64_t w0 = (uint64_t)t * kATile + (uint64_t)wave * kRegion;  // first element of this wave's region
     if (t == 0) {
         // the words the selection kernel accumulates into start every call at zero
