@@ -723,7 +723,7 @@ constexpr int kAWaves = kATile / kRegion;  // wavefronts (= regions) per streami
 constexpr int kAThreads = kAWaves * kWave;
 __global__ __launch_bounds__(kAThreads) void k_topk_pass_a_fast(Buckets, Geometry g, Workspace w) {
     const BucketsArg bk = buckets_arg();
-    __shared__ uint32_t stage[kAWaves][kRegSlots][2];
+    __shared__ __attribute__((aligned(16))) uint32_t stage[kAWaves][kRegSlots][2];
     const uint32_t b = blockIdx.y, t = blockIdx.x;
     const uint64_t bn = bucket_count(g, bk, b);
     const int lane = threadIdx.x & (kWave - 1);
@@ -762,43 +762,64 @@ __global__ __launch_bounds__(kAThreads) void k_topk_pass_a_fast(Buckets, Geometr
     issue(0);
     const Window wn = load_window(w.state + (uint64_t)b * kStateWords);
     const uint32_t lo_key = wn.lo, that_key = wn.that;
-    const uint64_t below = (1ull << lane) - 1ull;
-    uint32_t staged = 0;  // wave-uniform
-    bool dense = false;   // wave-uniform: more candidates than slots
+    // both the same in every lane, and kept in scalar registers by saying so at every update
+    uint32_t staged = 0;  // candidates of the region so far
+    uint32_t dense = 0;   // 1: more candidates than slots
+    u2a* const slots = (u2a*)&stage[wave][0][0];
+    // lanes of `m` below this one
+    auto lanes_below = [&](uint64_t m) {
+        return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+    };
+    auto pick = [](const u4a& a, uint32_t q) {
+        uint32_t v = a[0];
+        v = q == 1 ? a[1] : v;
+        v = q == 2 ? a[2] : v;
+        return q == 3 ? a[3] : v;
+    };
 
     // Appends the lanes' candidates (mask4: which of a lane's four elements) in
-    // index order: lane-major, element-minor.  `cnt` lanes-with-at-least-j
-    // ballots give every lane the number of candidates in the lanes below it.
+    // index order: lane-major, element-minor.  Nearly every call finds a few lanes
+    // with one candidate each: one ballot, one 8-byte LDS store.  Lanes with
+    // several candidates (about one call in ten has one) take the branch that
+    // counts them level by level and stores the rest in a loop.
     auto append = [&](uint32_t mask4, const u4a& a, uint32_t first_idx) {
+        const uint64_t m1 = __ballot(mask4 != 0);
+        if (!m1) return;  // wave-uniform
         const uint32_t c = __popc(mask4);
-        uint64_t m = __ballot(c >= 1);
-        if (!m) return;  // wave-uniform
-        uint32_t before = __popcll(m & below), total = __popcll(m);
-#pragma unroll
-        for (uint32_t level = 2; level <= 4; level++) {
-            m = __ballot(c >= level);
-            if (!m) break;  // wave-uniform; nearly always taken at level 2
-            before += __popcll(m & below);
-            total += __popcll(m);
+        uint32_t before = lanes_below(m1), total = __popcll(m1);
+        const uint64_t m2 = __ballot(c >= 2);
+        if (m2) {  // wave-uniform
+            before += lanes_below(m2);
+            total += __popcll(m2);
+            const uint64_t m3 = __ballot(c >= 3);
+            if (m3) {
+                const uint64_t m4 = __ballot(c >= 4);
+                before += lanes_below(m3) + lanes_below(m4);
+                total += __popcll(m3) + __popcll(m4);
+            }
         }
         if (dense) return;
+        total = (uint32_t)__builtin_amdgcn_readfirstlane((int)total);
         if (staged + total > (uint32_t)kRegSlots) {
             // the region goes dense: its earlier candidates were stored as zeros where
             // they reached the predicted threshold; put those values back
-            dense = true;
+            dense = 1u;
             if ((uint32_t)lane < staged && (stage[wave][lane][1] & 0x7FFFFFFFu) >= that_key)
                 bucket_residual(g, bk, b)[stage[wave][lane][0]] = u2f(stage[wave][lane][1]);
             return;
         }
-        uint32_t pos = staged + before;
-        while (mask4) {
+        if (mask4) {
+            uint32_t pos = staged + before;
             const uint32_t q = (uint32_t)__ffs((int)mask4) - 1u;
-            stage[wave][pos][0] = first_idx + q;
-            stage[wave][pos][1] = q == 0 ? a[0] : (q == 1 ? a[1] : (q == 2 ? a[2] : a[3]));
-            pos++;
-            mask4 &= mask4 - 1u;
+            slots[pos] = u2a{first_idx + q, pick(a, q)};
+            uint32_t rest = mask4 & (mask4 - 1u);
+            while (rest) {
+                const uint32_t q2 = (uint32_t)__ffs((int)rest) - 1u;
+                slots[++pos] = u2a{first_idx + q2, pick(a, q2)};
+                rest &= rest - 1u;
+            }
         }
-        staged += total;
+        staged = (uint32_t)__builtin_amdgcn_readfirstlane((int)(staged + total));
     };
 
 #pragma unroll
@@ -841,7 +862,7 @@ __global__ __launch_bounds__(kAThreads) void k_topk_pass_a_fast(Buckets, Geometr
     }
     const uint32_t region = (uint32_t)(w0 / kRegion);
     if (!dense && (uint32_t)lane < staged) {
-        u2a e = {stage[wave][lane][0], stage[wave][lane][1]};
+        const u2a e = slots[lane];
         *(u2a*)(w.list + (((uint64_t)b * g.regions + region) * kRegSlots + lane) * 2) = e;
     }
     if (lane == 0) w.reg_cnt[(uint64_t)b * g.regions + region] = dense ? kDense : staged;
