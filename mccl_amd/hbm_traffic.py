@@ -42,8 +42,10 @@ def per_kernel(path: str, counter: str) -> dict:
             if row["Counter_Name"] != counter:
                 continue
             name = row["Kernel_Name"]
-            for key in ("k_ring_fold", "k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail", "k_sparse_bounds",
-                        "k_sparse_accumulate", "copyBuffer"):
+            if "k_ring_fold" in name and "k_ring_fold<6, 0, true, 8>" not in name:
+                continue                                  # only the fp32 SUM fold of 8 ranks (config 2)
+            for key in ("k_ring_fold", "k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail", "k_sparse_starts",
+                        "k_sparse_bounds", "k_sparse_accumulate", "copyBuffer"):
                 if key in name:
                     vals[key].append((int(row["Grid_Size"]), float(row["Counter_Value"])))
                     break
@@ -88,7 +90,7 @@ def main(argv) -> int:
         "calls": {
             "ring_fold_f32_w8": total(["k_ring_fold"]),
             "topk_compress": total(["k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail"]),
-            "sparse_accumulate": total(["k_sparse_bounds", "k_sparse_accumulate"]),
+            "sparse_accumulate": total(["k_sparse_starts", "k_sparse_bounds", "k_sparse_accumulate"]),
         },
     }
     os.makedirs(os.path.dirname(OUT), exist_ok=True)
