@@ -194,3 +194,21 @@ def test_order_violation_at_any_position_is_flagged(ops, pos):
     idx, val = good[1][0][0].copy(), good[1][0][1]
     idx[k - 1] = n
     run_case(ops, [good[0], [(idx, val)]], n, n, None, expect_status=oracle.ERR_INDEX, paths=("auto",))
+
+
+def test_buckets_that_start_off_a_16_byte_boundary(ops):
+    # an odd bucket length puts every second bucket's first element off the vector alignment:
+    # those buckets' tiles take the element-wise write-out
+    rng = np.random.default_rng(77)
+    n, be, ws = 50_003, 10_001, 3
+    nb = (n + be - 1) // be
+    per_rank = []
+    for r in range(ws):
+        ranks = []
+        for b in range(nb):
+            bn = min(be, n - b * be)
+            k = max(1, bn // 50)
+            idx = np.sort(rng.choice(bn, size=k, replace=False)).astype(np.uint32)
+            ranks.append((idx, rng.standard_normal(k).astype(np.float32)))
+        per_rank.append(ranks)
+    run_case(ops, per_rank, n, be, 1.0 / 3.0)
