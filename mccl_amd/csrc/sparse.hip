@@ -517,7 +517,8 @@ __global__ __launch_bounds__(kRunWaves * kWave, 4) void k_sparse_accumulate_runs
         nreg[r] = kRunWins;
     }
 
-    for (uint32_t ts = (uint32_t)e0; ts < e1; ts += kRunL) {
+    for (uint64_t ts64 = e0; ts64 < e1; ts64 += kRunL) {  // 64-bit: the last tile of a 2^32-element bucket ends past 32 bits
+        const uint32_t ts = (uint32_t)ts64;
         const uint32_t tlen = (e1 - ts) < (uint32_t)kRunL ? (e1 - ts) : (uint32_t)kRunL;
         const uint32_t tend = ts + tlen;
 #pragma unroll
