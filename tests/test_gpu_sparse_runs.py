@@ -212,3 +212,30 @@ def test_buckets_that_start_off_a_16_byte_boundary(ops):
             ranks.append((idx, rng.standard_normal(k).astype(np.float32)))
         per_rank.append(ranks)
     run_case(ops, per_rank, n, be, 1.0 / 3.0)
+
+
+def test_random_shapes_and_payload_shapes(ops):
+    # seeded sweep: world size, bucket length (aligned or not), last bucket, density and clustering all vary
+    rng = np.random.default_rng(20260)
+    for case in range(40):
+        ws = int(rng.integers(1, 9))
+        be = int(rng.choice([1, 3, 64, 2047, 2048, 2049, 4096, 10_000, 33_333, 70_000]))
+        nb = int(rng.integers(1, 5))
+        n = max(1, be * (nb - 1) + int(rng.integers(1, be + 1)))
+        density = float(rng.choice([0.0005, 0.005, 0.01, 0.02, 0.04]))
+        per_rank = []
+        for r in range(ws):
+            ranks = []
+            for b in range((n + be - 1) // be):
+                bn = min(be, n - b * be)
+                k = min(bn, max(int(rng.integers(0, 2)), int(bn * density)))
+                if rng.random() < 0.3 and bn > 4 * max(k, 1):          # all pairs in one stretch of the bucket
+                    lo = int(rng.integers(0, bn - 2 * max(k, 1)))
+                    pool = np.arange(lo, lo + 2 * max(k, 1))
+                else:
+                    pool = bn
+                idx = np.sort(rng.choice(pool, size=k, replace=False)).astype(np.uint32)
+                ranks.append((idx, (rng.standard_normal(k) * 10.0 ** rng.integers(-20, 20)).astype(np.float32)))
+            per_rank.append(ranks)
+        scale = [None, 1.0 / ws, 0.3][case % 3]
+        run_case(ops, per_rank, n, be, scale, paths=("auto", None))
