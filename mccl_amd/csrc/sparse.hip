@@ -306,23 +306,26 @@ __global__ __launch_bounds__(kAccThreads) void k_sparse_accumulate_b(float* acc,
 // ---- runs of tiles, one wavefront each ------------------------------------------
 // The kernels above pay for finding where a tile's pairs begin: a table that a
 // pre-pass builds from a second read of every payload.  Here a wavefront owns a
-// run of consecutive 2048-element tiles of one bucket and walks every rank's
-// payload forward as it goes, so a position has to be found only where a run
-// begins, and only to the nearest 64 pairs: the wavefront keeps, for each rank,
-// a window of 64 consecutive pairs in registers (one per lane) plus the next
-// window, already requested.  A pair belongs to the current tile exactly when
-// its index lies inside it; pairs of earlier tiles are behind, pairs of later
-// tiles wait in the window.  When a window's last index is below the tile's end
-// the next window is swapped in and looked at for the same tile.  The tile sits
-// in LDS (8 KiB per wavefront), ranks add in ascending order (the LDS executes
-// one wavefront's operations in order, so no barrier is involved), and the tile
-// goes out once, scaled, in 16-byte stores.  Payload bytes are read once, plus
-// one window where two runs meet.
+// run of consecutive 2048-element tiles of one bucket (four tiles at 1 %
+// density) and needs a position only where its run begins, and only to the
+// nearest 64 pairs.  For each rank it requests three windows of 64 consecutive
+// pairs (one pair per lane) when the run begins, all ranks at once, and keeps
+// them in registers: every load of the run is issued before its first store
+// (a load after stores would wait for their acknowledgements).  A pair belongs
+// to the current tile exactly when its index lies inside it; pairs of earlier
+// tiles are behind, pairs of later tiles wait in their window.  When the
+// window's last index is below the tile's end the next window shifts in and is
+// looked at for the same tile; a run denser than its three windows fetches
+// further windows one at a time.  The tile sits in LDS (8 KiB per wavefront),
+// ranks add in ascending order (the LDS executes one wavefront's operations in
+// order, so no barrier is involved), and the tile goes out once, scaled, in
+// 16-byte stores.  Everything that decides control flow (tile bounds, window
+// ends, counts) lives in scalar registers.
 //
-// Where a run begins: k_sparse_starts reads one index per 64 pairs (an eighth of
-// the payload's cache lines) and writes, for every run w, the window that holds
-// the last sampled index below the run's first element; every pair before that
-// window belongs to an earlier run.
+// Where a run begins: k_sparse_starts reads every 64th index (one 128-byte line
+// in four) and writes, for every run w, the window that holds the last sampled
+// index below the run's first element; every pair before that window belongs to
+// an earlier run.
 constexpr int kRunL = 2048;    // elements per tile of a wavefront
 constexpr int kRunWaves = 4;   // wavefronts (= runs) per block
 constexpr int kRunRanks = 8;   // ranks a wavefront holds windows for; larger worlds use the tile kernels
@@ -394,7 +397,6 @@ __device__ __forceinline__ uint32_t window_index(u2a4 v, uint32_t base, uint32_t
     return base + (uint32_t)lane < k ? v[0] : 0xFFFFFFFFu;
 }
 
-// Indices of a window ascend, continue the pair before the window (`before`), and stay inside the bucket.
 // The value the lane below holds (lane 0: `first`): one DPP move, no LDS traffic.
 __device__ __forceinline__ uint32_t from_lane_below(uint32_t v, uint32_t first) {
     // wave_shr:1 - lane l reads lane l - 1 across the whole wavefront; lane 0 keeps `first`

@@ -10,12 +10,12 @@
 // `key = bits & 0x7FFFFFFF`, so selection is an exact radix select on that key.
 // All buckets of a gradient run in the same launches (blockIdx.y = bucket).
 //
-// FAST PATH (one pass over the gradient, 12 B/element of HBM traffic):
-//   sample     one block per bucket loads 12,288 evenly spread elements into
-//              LDS and radix-selects three of their keys: `lo`, which with 6 sigma
-//              of margin lies below the k-th largest key of the bucket, `hi`,
-//              which with the same margin lies above it, and the predicted
-//              threshold itself
+// FAST PATH (one pass over the gradient, 12 B/element of HBM traffic, three launches):
+//   sample     one block per bucket loads 12,288 evenly spread elements (keys
+//              stay in registers) and radix-selects three of their keys: `lo`,
+//              which with 6 sigma of margin lies below the k-th largest key of
+//              the bucket, `hi`, which with the same margin lies above it, and
+//              the predicted threshold itself
 //   pass A     residual <- grad + residual in one streaming pass, except that
 //              elements at or above the predicted threshold are stored as 0.0f
 //              at once; elements with key >= lo ("candidates", about 1.7 k) go,
@@ -23,21 +23,27 @@
 //              elements one wavefront streams): no atomics, no shared lists.
 //              A region with more than 64 candidates is marked dense and later
 //              read from the residual itself
-//   hist       256-bin histogram of the candidates, linear in the key over [lo, hi)
-//   select1    finds the histogram bin that holds the k-th largest key, counts
-//              per region the candidates in higher bins (picks for certain) and
-//              copies the threshold bin's candidates (a few hundred) to list2
-//   select2    one block per bucket: checks that the threshold lies inside the
-//              window (else the bucket is handed to the exact fallback, after
-//              the pre-zeroed values have been put back), finishes the radix
-//              select on list2: exact threshold key T, how many keys equal to T
-//              are taken and - when not all of them are - the largest index still
-//              taken; adds list2's picks to the region counts and scans them
-//              into each region's offset in the payload
-//   emit       an ordered filter: a wavefront per region writes the region's
-//              picks at its offset and repairs the residual where the predicted
-//              threshold and T disagree (zero a missed pick, restore a non-pick)
-// EXACT PATH (any input; also the per-bucket fallback of the fast path):
+//   selection  (k_topk_tail) 64 blocks per bucket that meet at two counter
+//              barriers; every wavefront keeps the slots of its regions in
+//              registers throughout.
+//              1: 256-bin histogram of the candidates, linear in the key over
+//                 [lo, hi)                                          -- barrier --
+//              2: the bin that holds the k-th largest key; per block the count
+//                 of candidates in higher bins (picks for certain); the
+//                 threshold bin's candidates (a few hundred) to list2
+//                                                                   -- barrier --
+//              3: every block finishes the radix select on list2: exact threshold
+//                 key T, how many keys equal to T are taken and - when not all of
+//                 them are - the largest index still taken
+//              4: an ordered filter: each block writes its regions' picks at its
+//                 offset in the payload (scan of the 64 blocks' counts) and
+//                 repairs the residual where the predicted threshold and T
+//                 disagree (zero a missed pick, restore a non-pick)
+//              A threshold outside the window, a list2 overflow or an
+//              inconsistent count hands the bucket to the exact fallback: its
+//              64 blocks put the pre-zeroed values back and run the radix
+//              select over the whole bucket together (three more barriers).
+// EXACT PATH (any input; small buckets and topk_path = 1):
 //   [pass A]   residual <- grad + residual, histogram of key[30:20]
 //   refine x2  histograms of key[19:10], key[9:0] among prefix matches
 //   count      per 4096-element tile: #(key > T), #(key == T)
