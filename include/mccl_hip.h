@@ -283,7 +283,8 @@ int mccl_hip_sync(void* stream);
 
 /* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
 /* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_warm", "topk_barrier_ms",
- * "sparse_path" (0 auto, 1 tile kernels only), "sparse_run_steps" (0 auto) */
+ * "sparse_path" (0 auto, 1 tile kernels only), "sparse_run_steps" (0 auto),
+ * "fp16_portable" (1: the casts follow the reference's portable branch, FP16Compression.cpp:38-73,:96-111) */
 int mccl_hip_set_tuning(const char* key, int value);
 int mccl_hip_get_tuning(const char* key);
 

@@ -145,6 +145,8 @@ int mccl_hip_set_tuning(const char* key, int value) {
     } else if (!std::strcmp(key, "topk_barrier_ms")) {
         if (value < 0 || value > 60000) return MCCL_HIP_ERR_ARG;
         t.topk_barrier_ms = value;
+    } else if (!std::strcmp(key, "fp16_portable")) {
+        t.fp16_portable = value ? 1 : 0;
     } else if (!std::strcmp(key, "sparse_path")) {
         if (value < 0 || value > 1) return MCCL_HIP_ERR_ARG;
         t.sparse_path = value;
@@ -165,6 +167,7 @@ int mccl_hip_get_tuning(const char* key) {
     if (!std::strcmp(key, "topk_path")) return t.topk_path;
     if (!std::strcmp(key, "topk_warm")) return t.topk_warm;
     if (!std::strcmp(key, "topk_barrier_ms")) return t.topk_barrier_ms;
+    if (!std::strcmp(key, "fp16_portable")) return t.fp16_portable;
     if (!std::strcmp(key, "sparse_path")) return t.sparse_path;
     if (!std::strcmp(key, "sparse_run_steps")) return t.sparse_run_steps;
     return MCCL_HIP_ERR_ARG;

@@ -119,3 +119,36 @@ class TestCompressor:
             c.decompress(wire, 7, dtype=torch.float16)
         with pytest.raises(RuntimeError, match="FP16 decompression only supports float32 output"):
             c.decompress(wire, 4, dtype=torch.bfloat16)
+
+
+needs_ref = pytest.mark.skipif(not oracle.RefCompressor.available(), reason="compiled reference not built")
+
+
+@needs_ref
+def test_portable_mode_is_the_compiled_reference_bit_for_bit():
+    # "fp16_portable" follows the branch of FP16Compression.cpp that a non-ARM build runs
+    # (:38-73, :96-111): checked against that very code, compiled from the reference's sources,
+    # over every half encoding, every rounding boundary and random bit patterns.
+    ref = oracle.RefCompressor(mode=1)
+    hip_ops.set_tuning("fp16_portable", 1)
+    try:
+        h = np.arange(65536, dtype=np.uint16)
+        got = to_np(hip_ops.cast_f16_to_f32(to_dev(h, oracle.F16)), oracle.F32)
+        want, rc = ref.decompress(h.view(np.uint8), h.size)
+        assert rc == 0 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        rng = np.random.default_rng(5)
+        rand = rng.integers(0, 1 << 32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        tiny = (rng.standard_normal(1 << 16) * 6e-5).astype(np.float32)          # around the smallest normal half
+        for x in (_boundary_inputs(), rand, tiny):
+            got = to_np(hip_ops.cast_f32_to_f16(to_dev(x, oracle.F32, pad_front=1)), oracle.F16)
+            want = ref.compress(x).view(np.uint16)
+            assert np.array_equal(got, want)
+        # the two modes differ exactly where the portable branch says they do
+        sub = np.array([1e-7, -3e-6, 6.0e-8, 6.2e-5, 6.1e-5], np.float32)        # 2^-14 = 6.1035e-5
+        flushed = to_np(hip_ops.cast_f32_to_f16(to_dev(sub, oracle.F32)), oracle.F16)
+        hip_ops.set_tuning("fp16_portable", 0)
+        kept = to_np(hip_ops.cast_f32_to_f16(to_dev(sub, oracle.F32)), oracle.F16)
+        assert list(flushed & 0x7FFF) == [0, 0, 0, int(kept[3] & 0x7FFF), 0] and all(kept & 0x7FFF)
+        assert list(flushed & 0x8000) == list(kept & 0x8000)
+    finally:
+        hip_ops.set_tuning("fp16_portable", 0)
