@@ -14,12 +14,12 @@
 //   runs of tiles (up to 8 ranks, payloads of the usual density, a workspace):
 //     one wavefront per run of 2048-element tiles, every rank's pairs held in
 //     registers, rank order kept by the LDS's in-order execution of one
-//     wavefront's adds; a small table says in which 64-pair window of each
+//     wavefront's adds; a small table says near which pair (to the nearest 80) of each
 //     payload a run begins.
 //   tile kernels (everything else): one block per 8192-element tile with a
 //     barrier between ranks, ranges from a bounds table or by binary search.
 // HBM traffic is close to the algorithmic minimum: every payload read once (plus
-// one index in 64 for the table), every output element written once.
+// one index in 80 for the table), every output element written once.
 #include "common.hip.h"
 #include "runtime.h"
 
@@ -308,7 +308,7 @@ __global__ __launch_bounds__(kAccThreads) void k_sparse_accumulate_b(float* acc,
 // pre-pass builds from a second read of every payload.  Here a wavefront owns a
 // run of consecutive 2048-element tiles of one bucket (four tiles at 1 %
 // density) and needs a position only where its run begins, and only to the
-// nearest 64 pairs.  For each rank it requests three windows of 64 consecutive
+// nearest 80 pairs.  For each rank it requests three windows of 64 consecutive
 // pairs (one pair per lane) when the run begins, all ranks at once, and keeps
 // them in registers: every load of the run is issued before its first store
 // (a load after stores would wait for their acknowledgements).  A pair belongs
@@ -322,21 +322,23 @@ __global__ __launch_bounds__(kAccThreads) void k_sparse_accumulate_b(float* acc,
 // 16-byte stores.  Everything that decides control flow (tile bounds, window
 // ends, counts) lives in scalar registers.
 //
-// Where a run begins: k_sparse_starts reads every 64th index (one 128-byte line
-// in four) and writes, for every run w, the window that holds the last sampled
+// Where a run begins: k_sparse_starts reads every 80th index (one 128-byte line
+// in five) and writes, for every run w, the window that holds the last sampled
 // index below the run's first element; every pair before that window belongs to
 // an earlier run.
 constexpr int kRunL = 2048;    // elements per tile of a wavefront (1024 and 4096 measured 4-5 % slower)
 constexpr int kRunWaves = 8;   // wavefronts (= runs) per block: 64 KiB of LDS, two blocks per CU (4 measured 3 % slower, 2 slower still)
 constexpr int kRunRanks = 8;   // ranks a wavefront holds windows for; larger worlds use the tile kernels
 constexpr int kWin = kWave;    // pairs per window
+constexpr int kStride = 80;    // pairs between two sampled indices of the position table: five 128-byte lines,
+                               // so a run begins with at most 79 pairs of an earlier run in its first window
 constexpr int kRunWins = 3;    // windows of a rank a wavefront requests when its run begins
 constexpr int kXcds = 8;       // accelerator dies of an MI355X; block B runs on die B mod 8
 
 constexpr int kStartThreads = 1024;
 constexpr uint32_t kStartSamples = 8192;  // samples of one payload the block keeps in LDS (32 KiB)
 
-// One block per (bucket, rank).  The samples (every 64th index) are requested before k is known
+// One block per (bucket, rank).  The samples (every 80th index) are requested before k is known
 // (inside the payload's capacity, masked afterwards), so the kernel is one round trip: samples
 // into LDS, then every run finds by binary search how many samples lie below its first element.
 __global__ __launch_bounds__(kStartThreads) void k_sparse_starts(WirePtrs wires, int ws, uint64_t wire_stride,
@@ -346,20 +348,20 @@ __global__ __launch_bounds__(kStartThreads) void k_sparse_starts(WirePtrs wires,
     const uint32_t b = blockIdx.x / (uint32_t)ws, r = blockIdx.x % (uint32_t)ws;
     const uint32_t* wp = (const uint32_t*)(wires.w[r] + (uint64_t)b * wire_stride);
     const uint32_t kmax = (uint32_t)((wire_stride - 4) / 8);
-    const uint32_t cap = (kmax + kWin - 1) / kWin;  // samples the payload can hold (at most kStartSamples)
+    const uint32_t cap = (kmax + kStride - 1) / kStride;  // samples the payload can hold (at most kStartSamples)
     constexpr int kPer = kStartSamples / kStartThreads;
     uint32_t v[kPer];
 #pragma unroll
     for (int i = 0; i < kPer; i++) {
         const uint32_t j = (uint32_t)i * kStartThreads + threadIdx.x;
-        v[i] = j < cap ? wp[1 + 2 * (uint64_t)kWin * j] : 0u;
+        v[i] = j < cap ? wp[1 + 2 * (uint64_t)kStride * j] : 0u;
     }
     uint32_t k = wp[0];
     if (k > kmax) {
         if (status) *status = MCCL_HIP_ERR_SIZE;
         k = 0;
     }
-    const uint32_t nsamp = (k + kWin - 1) / kWin;
+    const uint32_t nsamp = (k + kStride - 1) / kStride;
 #pragma unroll
     for (int i = 0; i < kPer; i++) {
         const uint32_t j = (uint32_t)i * kStartThreads + threadIdx.x;
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(kStartThreads) void k_sparse_starts(WirePtrs wires,
             if (samp[mid] < first) lo = mid + 1;
             else hi = mid;
         }
-        st[w] = lo ? (lo - 1) * kWin : 0u;
+        st[w] = lo ? (lo - 1) * kStride : 0u;
     }
 }
 
@@ -478,13 +480,13 @@ __global__ __launch_bounds__(kRunWaves * kWave, 4) void k_sparse_accumulate_runs
         }
 #pragma unroll
         for (int r = 0; r < NR; r++) {
-            uint32_t k = kraw[r], c = craw[r] & ~(uint32_t)(kWin - 1);
+            uint32_t k = kraw[r], c = craw[r];
             if (k > kmax) {
                 oversize = true;
                 k = 0;
             }
             if (r >= ws) k = 0;
-            if (c >= k) c = k ? ((k - 1) & ~(uint32_t)(kWin - 1)) : 0u;  // a table entry is never trusted
+            if (c >= k) c = k ? k - 1 : 0u;  // a table entry is never trusted
             kk[r] = __builtin_amdgcn_readfirstlane(k);
             wnext[r] = __builtin_amdgcn_readfirstlane(c);
         }
@@ -626,9 +628,10 @@ int accumulate(float* acc, uint64_t n_total, uint64_t bucket_elems, const void* 
     const uint64_t steps_bucket = (bucket_elems + kRunL - 1) / kRunL;
     const uint64_t per_tile = (kmax + steps_bucket - 1) / steps_bucket;
     if (ws <= kRunRanks && tuning().sparse_path != 1 && per_tile <= 96 && kmax >= 1 &&
-        (kmax + kWin - 1) / kWin <= kStartSamples) {
-        // a run is as many tiles as bring about 96 pairs of a rank, half of what the three windows
-        // requested at its start hold: a run of the usual density never loads again
+        (kmax + kStride - 1) / kStride <= kStartSamples) {
+        // a run is as many tiles as bring about 96 pairs of a rank: with up to 79 pairs of the run
+        // before it in the first window, the three windows requested at its start (192 pairs) hold a
+        // run of the usual density whole, and it never loads again
         uint64_t run_steps = (uint64_t)tuning().sparse_run_steps;
         if (run_steps == 0) run_steps = per_tile ? 96 / per_tile : 8;
         if (run_steps > 8 && tuning().sparse_run_steps == 0) run_steps = 8;
