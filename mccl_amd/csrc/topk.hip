@@ -55,6 +55,7 @@
 #include "common.hip.h"
 #include "runtime.h"
 
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -101,7 +102,8 @@ enum {
     S_DLO = 17,           // predicted threshold minus lower window end, in key units (from the last sample)
     S_DHI = 18,           // upper window end minus predicted threshold
     S_WARM = 19,          // 1 once a call has left a prediction behind
-    S_BARF = 20           // 20..23: barriers of the in-kernel exact selection
+    S_BARF = 20,          // 20..23: barriers of the in-kernel exact selection
+    S_READY = 24          // one-launch path: holds the launch's epoch number once the bucket's window is published
 };
 
 // The shared description of a bucket's window, and the rule every kernel applies to
@@ -148,6 +150,8 @@ struct Geometry {
     uint32_t regions;  // fast path: candidate regions allotted per bucket
     uint32_t lcap2;    // fast path: capacity of a bucket's list2 (entries)
     uint32_t listed;   // fast path: 1 when the buckets are separate buffers (see Buckets)
+    uint32_t ftiles;   // one-launch path: streaming tiles allotted per bucket
+    uint32_t lcapb;    // one-launch path: capacity of one coarse bin's list (entries)
 };
 
 struct Workspace {
@@ -163,6 +167,13 @@ struct Workspace {
     uint32_t* list2;        // [nbuckets][lcap2][2] candidates of the threshold bin (index, key)
     uint32_t* blk_above;    // [nbuckets][kNSub] fused tail: picks above the threshold bin per block
     uint32_t* blk_eq;       // [nbuckets][kNSub] in-kernel exact selection: keys equal to the threshold per block
+    // one-launch path
+    uint32_t* tile_cnt;     // [nbuckets][ftiles] candidates in the tile's slots, or kDense
+    uint64_t* slots;        // [nbuckets][ftiles][128] (bits << 32) | index, index order
+    uint32_t* grp_cnt;      // [nbuckets][64][kCntStride] finished tiles per group (first word of each 256 bytes)
+    uint32_t* ghist;        // [nbuckets][64 groups][64 bins] candidates per group and coarse window bin
+    uint32_t* bin_fill;     // [nbuckets][64] entries in each coarse bin's list
+    uint64_t* blist;        // [nbuckets][63][lcapb] the window's candidates by coarse bin, any order
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -1492,6 +1503,8 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Wo
     }
 }
 
+#include "topk_fused.hip.h"
+
 // ================================ host side =======================================
 
 uint64_t align4(uint64_t words) { return (words + 3) & ~uint64_t(3); }
@@ -1505,7 +1518,10 @@ uint64_t workspace_words(const Geometry& g) {
     return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) +
            align4((uint64_t)g.nbuckets * g.regions) +
            align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2) + align4((uint64_t)g.nbuckets * g.lcap2 * 2) +
-           2 * align4((uint64_t)g.nbuckets * kNSub);
+           2 * align4((uint64_t)g.nbuckets * kNSub) +
+           align4((uint64_t)g.nbuckets * g.ftiles) + align4((uint64_t)g.nbuckets * g.ftiles * kTileSlots * 2) +
+           align4((uint64_t)g.nbuckets * kGroups * kCntStride) + align4((uint64_t)g.nbuckets * kGroups * kCoarse) +
+           align4((uint64_t)g.nbuckets * kCoarse) + align4((uint64_t)g.nbuckets * (kCoarse - 1) * g.lcapb * 2);
 }
 
 Workspace carve(void* base, const Geometry& g) {
@@ -1520,7 +1536,13 @@ Workspace carve(void* base, const Geometry& g) {
     w.list = p;        p += align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2);
     w.list2 = p;       p += align4((uint64_t)g.nbuckets * g.lcap2 * 2);
     w.blk_above = p;   p += align4((uint64_t)g.nbuckets * kNSub);
-    w.blk_eq = p;
+    w.blk_eq = p;      p += align4((uint64_t)g.nbuckets * kNSub);
+    w.tile_cnt = p;    p += align4((uint64_t)g.nbuckets * g.ftiles);
+    w.slots = (uint64_t*)p;  p += align4((uint64_t)g.nbuckets * g.ftiles * kTileSlots * 2);
+    w.grp_cnt = p;     p += align4((uint64_t)g.nbuckets * kGroups * kCntStride);
+    w.ghist = p;       p += align4((uint64_t)g.nbuckets * kGroups * kCoarse);
+    w.bin_fill = p;    p += align4((uint64_t)g.nbuckets * kCoarse);
+    w.blist = (uint64_t*)p;
     return w;
 }
 
@@ -1543,11 +1565,42 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     if (cap > bucket_elems) cap = bucket_elems;
     g->lcap2 = (uint32_t)cap;
     g->listed = 0;
+    g->ftiles = (uint32_t)((bucket_elems + kFTile - 1) / kFTile);
+    // a coarse bin holds about k / 40 candidates when the window is as wide as a sample of
+    // 8192 leaves it; k / 8 + 2048 entries leave room for uneven bins
+    uint64_t capb = (uint64_t)g->k_full / 8 + 2048;
+    if (capb > bucket_elems) capb = bucket_elems;
+    g->lcapb = (uint32_t)capb;
     return true;
 }
 
-// The three launches of the single-pass path.
+std::atomic<uint32_t> g_epoch{0x5EED0001u};
+
+// The three launches of the single-pass path, or the one launch that does the same.
 void launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w, bool warm, hipStream_t st) {
+    // the streaming launch: a sample block per bucket, then per bucket its tiles and 64 bin blocks
+    const uint64_t blocks = (uint64_t)g.nbuckets * ((uint64_t)g.ftiles + kGroups + 1) + kGroups;
+    if (tuning().topk_fused && blocks < 0x7FFFFFFFull) {
+        uint32_t epoch = ++g_epoch;
+        if (epoch == 0) epoch = ++g_epoch;  // zero is what a finished call leaves in S_READY
+        // 100 MHz ticks a block may wait before it gives up
+        const uint64_t lim = (uint64_t)tuning().topk_barrier_ms * 100000ull;
+        // blocks that are resident from the start of the launch: they wait for the sample blocks
+        static const int per_cu = [] {
+            int n = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_topk_stream, kBlock, 0) != hipSuccess || n < 1) n = 5;
+            return n;
+        }();
+        const uint32_t first_wave = g.nbuckets + (uint32_t)device_info().num_cus * (uint32_t)per_cu;
+        k_topk_stream<<<(uint32_t)blocks, kBlock, 0, st>>>(bk, g, w, epoch, first_wave, lim);
+        // the select launch, at most kSelBuckets buckets at a time: all its blocks are resident
+        // together, whatever the order in which the hardware dispatches them
+        for (uint32_t b0 = 0; b0 < g.nbuckets; b0 += kSelBuckets) {
+            const uint32_t nb = g.nbuckets - b0 < (uint32_t)kSelBuckets ? g.nbuckets - b0 : (uint32_t)kSelBuckets;
+            k_topk_select<<<dim3(kGroups, nb), kBlock, 0, st>>>(bk, g, w, b0, lim);
+        }
+        return;
+    }
     // the window comes from the previous call's exact threshold when there was one
     if (!warm) k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(bk, g, w);
     const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
