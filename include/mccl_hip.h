@@ -157,16 +157,26 @@ uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, 
  * wire + b * wire_stride, and residual is zeroed at those elements.  Ties at
  * the threshold magnitude go to the lower index.  wire_stride must be a
  * multiple of 4 and at least 4 + 8 * k_b for the largest bucket
- * (else MCCL_HIP_ERR_CAPACITY).  NaN input is outside the contract. */
+ * (else MCCL_HIP_ERR_CAPACITY).
+ * Magnitudes are ordered by the bit pattern `bits & 0x7FFFFFFF`: infinities
+ * above every finite value, NaN patterns above infinity (by payload), ties to
+ * the lower index; a NaN gradient is therefore picked, sent and cleared from the
+ * residual like any other large value (the reference's comparator is undefined
+ * on NaN, TopKCompression.cpp:80-87).
+ * `status` (device int, may be null; the caller zeroes it) receives
+ * MCCL_HIP_ERR_TIMEOUT if a block of the single-pass path gave up waiting for
+ * another block of its launch (see "topk_barrier_ms"); the payload header of
+ * the bucket concerned is then 0xFFFFFFFF, which mccl_hip_topk_decompress and
+ * mccl_hip_sparse_accumulate reject with MCCL_HIP_ERR_SIZE. */
 int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
                            uint64_t bucket_elems, double ratio, void* wire,
                            uint64_t wire_stride, void* workspace, uint64_t workspace_bytes,
-                           void* stream);
+                           int* status, void* stream);
 
 /* TopKCompressor::compress for a LIST of buckets that are separate buffers of
  * their own lengths (the tensor list of a coalesced allreduce,
  * csrc/backend/ProcessGroupMCCL.cpp:2257-2313, compresses bucket by bucket), in
- * the same three launches as mccl_hip_topk_compress: per-bucket calls are bound
+ * the same two launches as mccl_hip_topk_compress: per-bucket calls are bound
  * by launch latency, a list is not.  host_grads[b] / host_residuals[b] hold
  * host_counts[b] fp32 elements; bucket b's payload [u32 k_b][k_b x {u32 index,
  * f32 value}] goes to host_wires[b], which holds host_wire_capacities[b] bytes
@@ -179,16 +189,7 @@ uint64_t mccl_hip_topk_list_workspace_bytes(const uint64_t* host_counts, uint32_
 int mccl_hip_topk_compress_list(const float* const* host_grads, float* const* host_residuals,
                                 const uint64_t* host_counts, void* const* host_wires,
                                 const uint64_t* host_wire_capacities, uint32_t nbuckets, double ratio,
-                                void* workspace, uint64_t workspace_bytes, void* stream);
-
-/* The workspace carries state from one call to the next: after a call it holds,
- * per bucket, the exact threshold just found, and the next call with the same
- * workspace and shape starts from it instead of sampling the gradient again (a
- * wrong prediction costs time, never correctness: the bucket is then selected
- * exactly).  Use one workspace per gradient tensor.  Call this before the memory
- * is freed or reused for something else, or to make the next call sample afresh.
- * No counterpart in the reference. */
-int mccl_hip_topk_workspace_forget(void* workspace);
+                                void* workspace, uint64_t workspace_bytes, int* status, void* stream);
 
 /* Diagnostics, no counterpart in the reference: after a compress call on
  * `stream` has been enqueued with this workspace and shape, waits for the
@@ -282,7 +283,7 @@ int mccl_hip_fence_block_stream(uint64_t ticket, void* stream);
 int mccl_hip_sync(void* stream);
 
 /* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
-/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_warm", "topk_barrier_ms",
+/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_barrier_ms",
  * "sparse_path" (0 auto, 1 tile kernels only), "sparse_run_steps" (0 auto),
  * "fp16_portable" (1: the casts follow the reference's portable branch, FP16Compression.cpp:38-73,:96-111) */
 int mccl_hip_set_tuning(const char* key, int value);

@@ -26,11 +26,10 @@ SIGNATURES = {
     "mccl_hip_topk_k": (_u32, [_u64, _f64]),
     "mccl_hip_topk_max_compressed_size": (_u64, [_u64, _f64]),
     "mccl_hip_topk_workspace_bytes": (_u64, [_u64, _u64, _f64]),
-    "mccl_hip_topk_compress": (_i32, [_vp, _vp, _u64, _u64, _f64, _vp, _u64, _vp, _u64, _vp]),
-    "mccl_hip_topk_workspace_forget": (_i32, [_vp]),
+    "mccl_hip_topk_compress": (_i32, [_vp, _vp, _u64, _u64, _f64, _vp, _u64, _vp, _u64, _vp, _vp]),
     "mccl_hip_topk_list_workspace_bytes": (_u64, [C.POINTER(_u64), _u32, _f64]),
     "mccl_hip_topk_compress_list": (_i32, [C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u64), C.POINTER(_vp),
-                                           C.POINTER(_u64), _u32, _f64, _vp, _u64, _vp]),
+                                           C.POINTER(_u64), _u32, _f64, _vp, _u64, _vp, _vp]),
     "mccl_hip_topk_path_report": (_i32, [_vp, _u64, _u64, _f64, C.POINTER(_u32), C.POINTER(_u32), _vp]),
     "mccl_hip_topk_decompress": (_i32, [_vp, _u64, _vp, _u64, _vp, _vp]),
     "mccl_hip_sparse_accumulate": (_i32, [_vp, _u64, _u64, C.POINTER(_vp), _i32, _u64, _i32, _f32, _vp, _vp, _u64, _vp]),

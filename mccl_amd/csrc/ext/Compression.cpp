@@ -93,6 +93,32 @@ at::Tensor& TopKCompressor::residual_for(uint64_t stable_id, size_t count) {
     return error_buffers_[stable_id];
 }
 
+// The device word the compress launches report a give-up through (a block of the single-pass
+// path that waited too long for another block of its launch).  The launches are asynchronous,
+// so the word is looked at by the calls that wait for the stream anyway: decompress() and
+// check_compress_status().  Caller holds mu_.
+int* TopKCompressor::compress_status() {
+    if (!compress_status_.defined())
+        compress_status_ = at::zeros({1}, at::TensorOptions().dtype(at::kInt).device(at::kCUDA));
+    return compress_status_.data_ptr<int>();
+}
+
+void TopKCompressor::throw_if_compress_failed() {
+    if (!compress_status_.defined()) return;
+    const int st = compress_status_.item<int>();
+    if (st == 0) return;
+    compress_status_.zero_();
+    if (st == MCCL_HIP_ERR_TIMEOUT)
+        throw TimeoutError("TopK compress: a block gave up waiting for another block of its launch; "
+                           "the payloads of that call are invalid");
+    throw_on_status(st, "TopK compress");
+}
+
+void TopKCompressor::check_compress_status() {
+    std::lock_guard<std::mutex> lock(mu_);
+    throw_if_compress_failed();
+}
+
 // One bucket on `stream`: csrc/compression/TopKCompression.cpp:38-120.  Caller holds mu_.
 size_t TopKCompressor::compress_on(const void* src, size_t nbytes, void* dst, size_t dst_capacity,
                                    at::Tensor& residual, at::Tensor& workspace, void* stream) {
@@ -104,13 +130,11 @@ size_t TopKCompressor::compress_on(const void* src, size_t nbytes, void* dst, si
         workspace = at::empty({static_cast<int64_t>(ws_bytes)},
                               at::TensorOptions().dtype(at::kByte).device(at::kCUDA));
     }
-    // the scratch is shared by buckets of different tensors: no threshold carried between calls
-    mccl_hip_topk_workspace_forget(workspace.data_ptr());
     // The payload's pairs start 4 bytes in; the stride only has to be a multiple of 4.
     const uint64_t stride = static_cast<uint64_t>(dst_capacity) & ~uint64_t(3);
     const int rc = mccl_hip_topk_compress(static_cast<const float*>(src), residual.data_ptr<float>(), count,
                                           count, k_ratio_, dst, stride, workspace.data_ptr(),
-                                          static_cast<uint64_t>(workspace.numel()), stream);
+                                          static_cast<uint64_t>(workspace.numel()), compress_status(), stream);
     if (rc == MCCL_HIP_ERR_CAPACITY) throw MCCLError("TopK compress: buffer too small");
     throw_on_status(rc, "TopK compress");
     MCCL_TRACE("TopK compress: %zu elements -> %u values, output %zu bytes", count, k, output_size);
@@ -158,7 +182,7 @@ std::vector<at::Tensor> TopKCompressor::compress_many(const std::vector<at::Tens
                    "compress_many: more distinct stable ids than the compressor holds residuals for");
         residuals.push_back(&it->second);
     }
-    // the list goes to the library in chunks of MCCL_HIP_TOPK_LIST_MAX buckets: three launches per chunk
+    // the list goes to the library in chunks of MCCL_HIP_TOPK_LIST_MAX buckets: two launches per chunk
     const int device = buckets[0].get_device();
     void* stream = c10::hip::getCurrentHIPStream(device).stream();
     std::vector<size_t> used(buckets.size());
@@ -182,7 +206,8 @@ std::vector<at::Tensor> TopKCompressor::compress_many(const std::vector<at::Tens
                                         at::TensorOptions().dtype(at::kByte).device(at::kCUDA));
         const int rc = mccl_hip_topk_compress_list(grads.data(), res.data(), counts.data(), wires.data(), caps.data(),
                                                    static_cast<uint32_t>(n), k_ratio_, list_workspace_.data_ptr(),
-                                                   static_cast<uint64_t>(list_workspace_.numel()), stream);
+                                                   static_cast<uint64_t>(list_workspace_.numel()), compress_status(),
+                                                   stream);
         if (rc == MCCL_HIP_ERR_CAPACITY) throw MCCLError("TopK compress: buffer too small");
         throw_on_status(rc, "TopK compress");
     }
@@ -207,6 +232,7 @@ void TopKCompressor::decompress(const void* src, size_t compressed_size, void* d
     if (rc == MCCL_HIP_ERR_SIZE) throw MCCLError("TopK decompress: size mismatch");
     throw_on_status(rc, "TopK decompress");
     const int st = status_.item<int>();
+    throw_if_compress_failed();
     if (st == MCCL_HIP_ERR_SIZE) throw MCCLError("TopK decompress: size mismatch");
     if (st == MCCL_HIP_ERR_INDEX) throw MCCLError("TopK decompress: index out of bounds");
 }

@@ -252,6 +252,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
            "Top-k payloads of a list of gradient buckets, one uint8 device tensor each")
         .def("reset_error_feedback", &mccl::TopKCompressor::reset_error_feedback)
         .def("reset_error_feedback_for_tensor", &mccl::TopKCompressor::reset_error_feedback_for_tensor)
+        .def("check_compress_status", &mccl::TopKCompressor::check_compress_status)
         .def("error_feedback_buffer_count", &mccl::TopKCompressor::error_feedback_buffer_count)
         .def("error_feedback_buffer", [](mccl::TopKCompressor& c, uint64_t id) -> py::object {
             at::Tensor t = c.error_feedback_buffer(id);

@@ -34,11 +34,16 @@ public:
     /// compress() for a list of buckets (float32 device tensors, one stable id each), the shape
     /// of a coalesced allreduce (csrc/backend/ProcessGroupMCCL.cpp:2257-2313 walks its tensor
     /// list bucket by bucket).  Returns one payload tensor per bucket, identical to what the
-    /// per-bucket calls give.  A bucket's three launches are latency-bound (and fifteen calls
-    /// are bound by the host's launch rate), so the whole list goes through the same three
-    /// launches (mccl_hip_topk_compress_list).
+    /// per-bucket calls give.  A bucket's launches are latency-bound (and fifteen calls are
+    /// bound by the host's launch rate), so the whole list goes through the same two launches
+    /// (mccl_hip_topk_compress_list).
     std::vector<at::Tensor> compress_many(const std::vector<at::Tensor>& buckets,
                                           const std::vector<uint64_t>& stable_ids);
+
+    /// Waits for the stream and throws TimeoutError if a compress launch since the last check
+    /// gave up (its payload headers then hold 0xFFFFFFFF and decompress rejects them).  No
+    /// counterpart in the reference, whose compress is synchronous host code.
+    void check_compress_status();
 
     double k_ratio() const { return k_ratio_; }
 
@@ -50,6 +55,9 @@ private:
     at::Tensor workspace_;       // scratch of a one-bucket call
     at::Tensor list_workspace_;  // scratch of a list call
     at::Tensor status_;  // device int32[1], written by decompress
+    at::Tensor compress_status_;  // device int32[1], written by a compress launch that gives up
+    int* compress_status();
+    void throw_if_compress_failed();
     at::Tensor& residual_for(uint64_t stable_id, size_t count);
     size_t compress_on(const void* src, size_t nbytes, void* dst, size_t dst_capacity, at::Tensor& residual,
                        at::Tensor& workspace, void* stream);

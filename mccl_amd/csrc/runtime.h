@@ -22,9 +22,7 @@ struct Tuning {
     int fold_blocks_per_cu = 256;  // grid cap of the streaming kernels, in blocks per CU
     int nontemporal = 1;         // 1: streaming loads/stores carry the `nt` hint (+8..12 % on MI355X)
     int topk_path = 0;           // 0 auto, 1 multi-pass exact path only, 2 single-pass path at any size
-    int topk_warm = 0;           // single-pass path: 1 start from the previous call's threshold instead of a sample (stationary gradients only)
-    int topk_fused = 1;          // single-pass path: 1 = one launch, 0 = three launches
-    int topk_barrier_ms = 2000;  // fused tail: longest wait of a block at a bucket barrier
+    int topk_barrier_ms = 2000;  // single-pass path: longest wait of a block for another block of its launch
     int fp16_portable = 0;       // FP16 casts: 1 = the reference's portable branch (half subnormals flushed, NaN bits passed through)
     int sparse_path = 0;         // sparse accumulate with a workspace: 0 auto (runs of tiles up to 8 ranks), 1 tile kernels only
     int sparse_run_steps = 0;    // runs of tiles: 2048-element tiles per wavefront, 0 = from the input's size

@@ -6,44 +6,14 @@
 // residual = adjusted everywhere except 0.0f at the picks.  Ties at the
 // threshold magnitude go to the lower index.
 //
-// For non-NaN floats, ordering by fabs() is ordering of the 31-bit pattern
-// `key = bits & 0x7FFFFFFF`, so selection is an exact radix select on that key.
-// All buckets of a gradient run in the same launches (blockIdx.y = bucket).
+// Ordering by fabs() is ordering of the 31-bit pattern `key = bits & 0x7FFFFFFF`
+// (NaN patterns sort above infinity), so selection is an exact radix select on
+// that key.  All buckets of a gradient run in the same launches.
 //
-// FAST PATH (one pass over the gradient, 12 B/element of HBM traffic, three launches):
-//   sample     one block per bucket loads 12,288 evenly spread elements (keys
-//              stay in registers) and radix-selects three of their keys: `lo`,
-//              which with 6 sigma of margin lies below the k-th largest key of
-//              the bucket, `hi`, which with the same margin lies above it, and
-//              the predicted threshold itself
-//   pass A     residual <- grad + residual in one streaming pass, except that
-//              elements at or above the predicted threshold are stored as 0.0f
-//              at once; elements with key >= lo ("candidates", about 1.7 k) go,
-//              in index order, to the 64 slots of their region (the 2048
-//              elements one wavefront streams): no atomics, no shared lists.
-//              A region with more than 64 candidates is marked dense and later
-//              read from the residual itself
-//   selection  (k_topk_tail) 64 blocks per bucket that meet at two counter
-//              barriers; every wavefront keeps the slots of its regions in
-//              registers throughout.
-//              1: 256-bin histogram of the candidates, linear in the key over
-//                 [lo, hi)                                          -- barrier --
-//              2: the bin that holds the k-th largest key; per block the count
-//                 of candidates in higher bins (picks for certain); the
-//                 threshold bin's candidates (a few hundred) to list2
-//                                                                   -- barrier --
-//              3: every block finishes the radix select on list2: exact threshold
-//                 key T, how many keys equal to T are taken and - when not all of
-//                 them are - the largest index still taken
-//              4: an ordered filter: each block writes its regions' picks at its
-//                 offset in the payload (scan of the 64 blocks' counts) and
-//                 repairs the residual where the predicted threshold and T
-//                 disagree (zero a missed pick, restore a non-pick)
-//              A threshold outside the window, a list2 overflow or an
-//              inconsistent count hands the bucket to the exact fallback: its
-//              64 blocks put the pre-zeroed values back and run the radix
-//              select over the whole bucket together (three more barriers).
-// EXACT PATH (any input; small buckets and topk_path = 1):
+// SINGLE-PASS PATH (one pass over the gradient, 12 B/element of HBM traffic, two
+// launches; default for buckets of 2^18 elements and more): see the section
+// "single-pass path" below.
+// EXACT PATH (any input; small buckets and topk_path = 1; six launches):
 //   [pass A]   residual <- grad + residual, histogram of key[30:20]
 //   refine x2  histograms of key[19:10], key[9:0] among prefix matches
 //   count      per 4096-element tile: #(key > T), #(key == T)
@@ -56,8 +26,6 @@
 #include "runtime.h"
 
 #include <atomic>
-#include <mutex>
-#include <unordered_map>
 #include <vector>
 
 namespace mcclhip {
@@ -67,78 +35,27 @@ namespace {
 constexpr int kTile = 4096;    // exact path: elements per compaction tile
 constexpr int kBins0 = 2048;   // key[30:20]
 constexpr int kBinsR = 1024;   // key[19:10], key[9:0]
-constexpr int kWinBins = 256;  // fast path: bins of the candidate window histogram
 constexpr int kHistWords = kBins0 + 2 * kBinsR;
 constexpr int kStateWords = 32;
-constexpr int kATile = 8192;   // fast path: elements per pass-A block
-constexpr int kRegion = 2048;  // fast path: elements per candidate region (one wavefront of a pass-A block)
-constexpr int kRegSlots = 64;  // fast path: candidate slots per region, one per lane of the wavefront that reads it
-static_assert(kATile == kRegion * (kBlock / kWave), "one region per wavefront");
-static_assert(kRegSlots == kWave, "a wavefront reads a region's slots in one go");
-constexpr uint32_t kDense = 0xFFFFFFFFu;  // region count: more candidates than slots, read the residual range itself
-constexpr int kNSub = 64;      // fast path: blocks per bucket in the kernels that walk the regions
-constexpr int kSampleThreads = 1024;  // sample kernel (256 threads measured slower: 21 vs 15.5 us)
+constexpr uint32_t kDense = 0xFFFFFFFFu;  // tile count: more candidates than slots, read the residual range itself
 constexpr uint64_t kFastMinBucket = 1u << 18;
-constexpr int kSample = 12288;  // fast path: sampled elements per bucket (12 per select thread)
 
 // per-bucket state words
 enum {
-    S_P0 = 0, S_R0 = 1,   // key prefix / picks still to place after round 0
-    S_P1 = 2, S_R1 = 3,   // after round 1
-    S_T = 4, S_NEED = 5,  // exact threshold key, number of keys == T that are taken
-    S_LO_KEY = 6,         // fast path: candidates have key >= this
-    S_HI_KEY = 11,        // fast path: keys >= this fall into the top bin of the window histogram
-    S_SHIFT = 12,         // fast path: window bin = (key - lo) >> shift
-    S_OK = 7,             // fast path: 1 when select succeeded for this bucket
-    S_ISTAR = 8,          // fast path: ties are taken while index <= this
-    S_EXACT_HIST = 9,     // 1 when hist round 0 holds the full histogram
-    S_N2 = 10,            // fast path: entries in list2
-    S_THAT = 13,          // fast path: predicted threshold key; pass A stores 0 for keys >= this
-    S_BAR1 = 14,          // fused tail: blocks of the bucket that have flushed their histogram
-    S_BAR2 = 15,          // fused tail: blocks that have published their certain picks and list2 share
-    S_TIMEOUT = 16,       // fused tail: a block gave up waiting at a barrier (result invalid)
-    // The window words (S_LO_KEY, S_HI_KEY, S_SHIFT, S_THAT) and the next three survive from
-    // call to call: after every call they hold the window predicted for the next one.
-    S_DLO = 17,           // predicted threshold minus lower window end, in key units (from the last sample)
-    S_DHI = 18,           // upper window end minus predicted threshold
-    S_WARM = 19,          // 1 once a call has left a prediction behind
-    S_BARF = 20,          // 20..23: barriers of the in-kernel exact selection
-    S_READY = 24          // one-launch path: holds the launch's epoch number once the bucket's window is published
+    // single-pass path: the candidate window, published by its sample block with ONE 16-byte store
+    S_LO_KEY = 0,         // candidates have key >= this
+    S_HI_KEY = 1,         // keys >= this fall into the top coarse bin
+    S_THAT = 2,           // predicted threshold key; the streaming blocks store 0.0f for keys >= this
+    S_READY = 3,          // the call's epoch number once the other three are valid; 0 after the call
+    S_P0 = 4, S_R0 = 5,   // exact path: key prefix / picks still to place after round 0
+    S_P1 = 6, S_R1 = 7,   // after round 1
+    S_T = 8, S_NEED = 9,  // exact threshold key, number of keys == T that are taken
+    S_ISTAR = 10,         // single-pass path: ties are taken while index <= this
+    S_OK = 11,            // single-pass path: 1 when the window selection succeeded for this bucket
+    S_EXACT_HIST = 12,    // 1 when hist round 0 holds the full histogram
+    S_TIMEOUT = 13,       // single-pass path: a block gave up waiting (result invalid, payload header poisoned)
+    S_BARF = 16           // 16..19: barriers of the exact selection inside the select launch
 };
-
-// The shared description of a bucket's window, and the rule every kernel applies to
-// whatever the state words hold (they may be stale or arbitrary when a caller hands
-// in a workspace with foreign contents): elements are only ever stored as zero when
-// they are also listed, i.e. the predicted threshold is never below the window.
-struct Window {
-    uint32_t lo, hi, shift, that;
-    bool sound;  // bins fit the histogram; otherwise the bucket takes the exact selection
-};
-__device__ __forceinline__ Window load_window(const uint32_t* st) {
-    Window wn;
-    wn.lo = st[S_LO_KEY];
-    wn.hi = st[S_HI_KEY];
-    wn.shift = st[S_SHIFT];
-    wn.that = st[S_THAT] < wn.lo ? wn.lo : st[S_THAT];
-    wn.sound = wn.shift < 32u && wn.hi >= wn.lo && ((wn.hi - wn.lo) >> (wn.shift & 31u)) < (uint32_t)(kWinBins - 1);
-    wn.shift &= 31u;
-    return wn;
-}
-// Block (0, b) of a call's last kernel: the window for the next call, centred on this call's
-// exact threshold with the widths the last sample found.
-__device__ __forceinline__ void predict_next_window(uint32_t* st, uint32_t T) {
-    const uint32_t dlo = st[S_DLO], dhi = st[S_DHI];
-    const uint32_t lo = T > dlo ? T - dlo : 0u;
-    uint32_t hi = dhi < 0x7FFFFFFFu - T ? T + dhi : 0x7FFFFFFFu;
-    if (hi < lo) hi = lo;
-    uint32_t shift = 0;
-    while (((hi - lo) >> shift) >= (uint32_t)(kWinBins - 1)) shift++;
-    st[S_LO_KEY] = lo;
-    st[S_HI_KEY] = hi;
-    st[S_SHIFT] = shift;
-    st[S_THAT] = T < lo ? lo : T;
-    st[S_WARM] = 1u;
-}
 
 struct Geometry {
     uint64_t n_total;
@@ -147,33 +64,28 @@ struct Geometry {
     uint32_t tiles;    // exact-path tiles per (full) bucket
     uint32_t k_full;   // k of a bucket with bucket_elems elements
     uint32_t k_last;   // k of the last bucket
-    uint32_t regions;  // fast path: candidate regions allotted per bucket
-    uint32_t lcap2;    // fast path: capacity of a bucket's list2 (entries)
-    uint32_t listed;   // fast path: 1 when the buckets are separate buffers (see Buckets)
-    uint32_t ftiles;   // one-launch path: streaming tiles allotted per bucket
-    uint32_t lcapb;    // one-launch path: capacity of one coarse bin's list (entries)
+    uint32_t listed;   // single-pass path: 1 when the buckets are separate buffers (see Buckets)
+    uint32_t ftiles;   // single-pass path: streaming tiles allotted per bucket
+    uint32_t lcapb;    // single-pass path: capacity of one coarse bin's list (entries)
 };
 
 struct Workspace {
     // zeroed at the start of every exact-path call; the single-pass path zeroes what it uses itself
     uint32_t* hist;         // [nbuckets][kHistWords]
-    uint32_t* hist_w;       // [nbuckets][kWinBins] candidates: window histogram, last bin = above the window
     uint32_t* state;        // [nbuckets][kStateWords]
     // scratch, written before read
     uint32_t* tile_gt;      // [nbuckets][tiles]
     uint32_t* tile_eq;      // [nbuckets][tiles]
-    uint32_t* reg_cnt;      // [nbuckets][regions] candidates in the region's slots, or kDense
-    uint32_t* list;         // [nbuckets][regions][kRegSlots][2]  (index, bits), index order
-    uint32_t* list2;        // [nbuckets][lcap2][2] candidates of the threshold bin (index, key)
-    uint32_t* blk_above;    // [nbuckets][kNSub] fused tail: picks above the threshold bin per block
-    uint32_t* blk_eq;       // [nbuckets][kNSub] in-kernel exact selection: keys equal to the threshold per block
-    // one-launch path
+    uint32_t* blk_above;    // [nbuckets][64] exact selection inside the select launch: keys above the threshold per group
+    uint32_t* blk_eq;       // [nbuckets][64] ... keys equal to the threshold per group
+    // single-pass path
     uint32_t* tile_cnt;     // [nbuckets][ftiles] candidates in the tile's slots, or kDense
     uint64_t* slots;        // [nbuckets][ftiles][128] (bits << 32) | index, index order
     uint32_t* grp_cnt;      // [nbuckets][64][kCntStride] finished tiles per group (first word of each 256 bytes)
     uint32_t* ghist;        // [nbuckets][64 groups][64 bins] candidates per group and coarse window bin
     uint32_t* bin_fill;     // [nbuckets][64] entries in each coarse bin's list
     uint64_t* blist;        // [nbuckets][63][lcapb] the window's candidates by coarse bin, any order
+    int* status;            // caller's device word (may be null): receives MCCL_HIP_ERR_TIMEOUT when a block gives up
 };
 
 __device__ __forceinline__ uint64_t bucket_count(const Geometry& g, uint32_t b) {
@@ -583,326 +495,7 @@ __global__ __launch_bounds__(kBlock) void k_topk_emit(float* residual, Geometry 
     }
 }
 
-// ================================= fast path ======================================
-
-// Window bin of a candidate key: linear in the key over [lo, hi), everything
-// at or above hi in bin kWinBins - 1.
-__device__ __forceinline__ uint32_t window_bin(uint32_t key, uint32_t lo, uint32_t hi, uint32_t shift) {
-    return key >= hi ? (uint32_t)(kWinBins - 1) : (key - lo) >> shift;
-}
-
-// One block per bucket.  Loads kSample evenly spread elements of grad + residual
-// (their keys stay in registers, 12 per thread) and radix-selects (11 + 10 key
-// bits, all ranks in the same sweeps) the keys of sample ranks
-//     r_hi = ks - 6 sqrt(ks) - 16,   r_lo = ks + 6 sqrt(ks) + 16   and   ks,
-// ks = k * S / n being the expected number of sampled elements among the top k:
-// the two ends of the candidate window and the predicted threshold.
-__global__ __launch_bounds__(kSampleThreads) void k_topk_sample(Buckets, Geometry g, Workspace w) {
-    const BucketsArg bk = buckets_arg();
-    __shared__ uint32_t lh[3][kBinsR];
-    __shared__ uint32_t scratch[3 * (kSampleThreads / kWave + 2)];
-    const uint32_t b = blockIdx.x;
-    const uint64_t bn = bucket_count(g, bk, b);
-    const float* gp = bucket_grad(g, bk, b);
-    const float* rp = bucket_residual(g, bk, b);
-    const uint64_t nvec = bn / 4;
-    constexpr int SV = kSample / 4;               // sampled vectors
-    constexpr int PV = SV / kSampleThreads;       // vectors per thread; their 4 * PV keys stay in registers
-    // sampled in runs of 8 vectors (one 128-byte line per array), runs evenly spread
-    const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)(nvec & ~7ull) : (uint32_t)SV;
-    const uint64_t stride = nsv ? (nvec / (nsv / 8)) : 8;  // vectors between run starts (>= 8)
-    u4a gv[PV], rv[PV];
-#pragma unroll
-    for (int j = 0; j < PV; j++) {
-        const uint32_t i = (uint32_t)j * kSampleThreads + threadIdx.x;
-        const uint32_t ii = i < nsv ? i : 0;
-        const uint64_t v = (uint64_t)(ii >> 3) * stride + (ii & 7);
-        gv[j] = nsv ? *(const u4u4*)(gp + v * 4) : u4a{0u, 0u, 0u, 0u};
-        rv[j] = nsv ? *(const u4u4*)(rp + v * 4) : u4a{0u, 0u, 0u, 0u};
-    }
-    // the histogram is cleared while the loads are under way
-    for (int i = threadIdx.x; i < 3 * kBinsR; i += kSampleThreads) (&lh[0][0])[i] = 0;
-    uint32_t key[PV][4];
-    bool have[PV];
-#pragma unroll
-    for (int j = 0; j < PV; j++) {
-        have[j] = (uint32_t)j * kSampleThreads + threadIdx.x < nsv;
-#pragma unroll
-        for (int q = 0; q < 4; q++) key[j][q] = key_of(u2f(gv[j][q]) + u2f(rv[j][q]));
-    }
-    const uint32_t S = nsv * 4;
-    const float ks = (float)bucket_k(g, bk, b) * (float)S / (float)bn;
-    const float margin = 6.0f * sqrtf(ks) + 16.0f;
-    // ranks: 0 upper end of the window, 1 lower end, 2 the predicted threshold itself
-    constexpr int NR = 3;
-    uint32_t rank[NR];
-    rank[0] = ks - margin >= 1.0f ? (uint32_t)(ks - margin) : 0u;  // 0: no upper end
-    rank[1] = (uint32_t)(ks + margin) + 1u;                       // > S: no lower end
-    rank[2] = ks >= 1.0f ? (uint32_t)ks : 1u;
-    uint32_t prefix[NR] = {0u, 0u, 0u}, want[NR] = {rank[0], rank[1], rank[2]};
-    const bool active[NR] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S, rank[2] <= S};
-    // Two rounds, 11 + 10 key bits: the selected keys are exact to 2^-13 of their value,
-    // far finer than the sampling noise the window margins allow for.  The ten low bits
-    // are filled so that the window only widens.
-    __syncthreads();
-    for (int r = 0; r < 2; r++) {
-        // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent, one histogram serves all ranks
-        uint32_t* h0 = &lh[0][0];
-        if (r == 1) {
-            for (int i = threadIdx.x; i < NR * kBinsR; i += kSampleThreads) h0[i] = 0;
-            __syncthreads();
-        }
-#pragma unroll
-        for (int j = 0; j < PV; j++) {
-            if (!have[j]) continue;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const uint32_t kq = key[j][q];
-                if (r == 0) {
-                    atomicAdd(&h0[kq >> 20], 1u);
-                } else {
-#pragma unroll
-                    for (int z = 0; z < NR; z++)
-                        if (active[z] && (kq >> 20) == (prefix[z] >> 20)) atomicAdd(&lh[z][(kq >> 10) & (kBinsR - 1)], 1u);
-                }
-            }
-        }
-        __syncthreads();
-        uint32_t rem[NR], bin[NR], left[NR];
-#pragma unroll
-        for (int z = 0; z < NR; z++) rem[z] = active[z] ? want[z] : 0u;
-        if (r == 0) {
-            const uint32_t* const hs[NR] = {h0, h0, h0};
-            pick_bins<kBins0, kSampleThreads, NR>(hs, rem, bin, left, scratch);
-        } else {
-            const uint32_t* const hs[NR] = {lh[0], lh[1], lh[2]};
-            pick_bins<kBinsR, kSampleThreads, NR>(hs, rem, bin, left, scratch);
-        }
-#pragma unroll
-        for (int z = 0; z < NR; z++) {
-            if (!active[z]) continue;
-            prefix[z] |= bin[z] << (r == 0 ? 20 : 10);
-            want[z] = left[z];
-        }
-    }
-    prefix[0] |= 0x3FFu;  // upper end of the window: rounded up
-    prefix[2] |= 0x200u;  // predicted threshold: middle of its 1024-key cell
-    if (threadIdx.x == 0) {
-        const uint32_t lo = active[1] ? prefix[1] : 0u;
-        uint32_t hi = active[0] ? prefix[0] : 0x7FFFFFFFu;
-        if (hi < lo) hi = lo;
-        uint32_t shift = 0;
-        while (((hi - lo) >> shift) >= (uint32_t)(kWinBins - 1)) shift++;
-        uint32_t* st = w.state + (uint64_t)b * kStateWords;
-        st[S_LO_KEY] = lo;
-        st[S_HI_KEY] = hi;
-        st[S_SHIFT] = shift;
-        // never below lo: every pre-zeroed element must be a listed candidate
-        uint32_t that = active[2] ? prefix[2] : 0x7FFFFFFFu;
-        if (that < lo) that = lo;
-        st[S_THAT] = that;
-        // widths for the predictions that follow this call
-        st[S_DLO] = that - lo;
-        st[S_DHI] = hi > that ? hi - that : 0u;
-        st[S_WARM] = 1u;
-    }
-}
-
-// ---- candidate regions ------------------------------------------------------------
-// A region is the kRegion consecutive elements one wavefront of a pass-A block
-// streams.  Its candidates land, in index order, in the region's kRegSlots slots
-// of `list` (slot = lane of the wave that later reads it) and their number in
-// reg_cnt.  A region with more candidates than slots is marked kDense: readers
-// then take every element of the region's residual range as a candidate.  No
-// atomics and no shared capacity are involved, so nothing can overflow.
-
-// The regions [r0, r1) of bucket b that block s of kNSub works on.
-__device__ __forceinline__ void block_regions(const Geometry& g, BucketsArg bk, uint32_t b, uint32_t s,
-                                              uint32_t* r0, uint32_t* r1) {
-    const uint32_t nreg = (uint32_t)((bucket_count(g, bk, b) + kRegion - 1) / kRegion);
-    const uint32_t per = (nreg + kNSub - 1) / kNSub;
-    *r0 = s * per < nreg ? s * per : nreg;
-    *r1 = *r0 + per < nreg ? *r0 + per : nreg;
-}
-
-// residual <- grad + residual; candidates (key >= lo) are written to their
-// region.  One 8192-element tile per block, tiles in address order, one region
-// per wavefront.  Elements at or above the predicted threshold are stored as
-// 0.0f straight away (their values are in the region's list): a million
-// scattered 4-byte stores after the selection cost more than a tenth of the
-// whole compress, while the streaming store here is free; emit only repairs
-// the few elements between the predicted and the true threshold.  A region
-// that turns out dense puts its values back and stores plain sums from then on.
-// Nothing else happens here: returning atomics and histogram flushes in these
-// 12,000 streaming blocks each cost 7-15 % of the kernel's time when they were
-// tried.
-constexpr int kAWaves = kATile / kRegion;  // wavefronts (= regions) per streaming block; 1, 2 and 8 measured the same or worse
-constexpr int kAThreads = kAWaves * kWave;
-__global__ __launch_bounds__(kAThreads) void k_topk_pass_a_fast(Buckets, Geometry g, Workspace w) {
-    const BucketsArg bk = buckets_arg();
-    __shared__ __attribute__((aligned(16))) uint32_t stage[kAWaves][kRegSlots][2];
-    const uint32_t b = blockIdx.y, t = blockIdx.x;
-    const uint64_t bn = bucket_count(g, bk, b);
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
-    const uint64_t w0 = (uint64_t)t * kATile + (uint64_t)wave * kRegion;  // first element of this wave's region
-    if (t == 0) {
-        // the words the selection kernel accumulates into start every call at zero
-        for (int i = threadIdx.x; i < kWinBins; i += kAThreads) w.hist_w[(uint64_t)b * kWinBins + i] = 0;
-        if (threadIdx.x == 0) {
-            uint32_t* st = w.state + (uint64_t)b * kStateWords;
-            st[S_BAR1] = 0; st[S_BAR2] = 0; st[S_N2] = 0; st[S_OK] = 0; st[S_TIMEOUT] = 0;
-            st[S_BARF] = 0; st[S_BARF + 1] = 0; st[S_BARF + 2] = 0; st[S_BARF + 3] = 0;
-        }
-        for (int i = threadIdx.x; i < kHistWords; i += kAThreads) w.hist[(uint64_t)b * kHistWords + i] = 0;
-    }
-    if (w0 >= bn) return;  // whole wavefront; the kernel has no barriers
-    const float* gp = bucket_grad(g, bk, b) + w0;
-    float* rp = bucket_residual(g, bk, b) + w0;
-    constexpr int U = 2;
-    constexpr int ROUNDS = kRegion / (kWave * 4 * U);
-    const uint32_t len = (uint32_t)((bn - w0) < (uint64_t)kRegion ? (bn - w0) : (uint64_t)kRegion);
-    const uint32_t nfull = len / 4;  // full vectors in this region
-    // The streaming loads of a round are issued one round ahead: round 0's before
-    // the bucket parameters are read, round r+1's before round r is processed.
-    u4a gv[ROUNDS][U], rv[ROUNDS][U];
-    auto issue = [&](int round) {
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t vi = (uint32_t)(round * U + u) * kWave + lane;
-            if (vi < nfull) {
-                gv[round][u] = __builtin_nontemporal_load((const u4u4*)(gp + vi * 4));
-                rv[round][u] = __builtin_nontemporal_load((const u4u4*)(rp + vi * 4));
-            }
-        }
-    };
-    issue(0);
-    const Window wn = load_window(w.state + (uint64_t)b * kStateWords);
-    const uint32_t lo_key = wn.lo, that_key = wn.that;
-    // both the same in every lane, and kept in scalar registers by saying so at every update
-    uint32_t staged = 0;  // candidates of the region so far
-    uint32_t dense = 0;   // 1: more candidates than slots
-    u2a* const slots = (u2a*)&stage[wave][0][0];
-    // lanes of `m` below this one
-    auto lanes_below = [&](uint64_t m) {
-        return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-    };
-    auto pick = [](const u4a& a, uint32_t q) {
-        uint32_t v = a[0];
-        v = q == 1 ? a[1] : v;
-        v = q == 2 ? a[2] : v;
-        return q == 3 ? a[3] : v;
-    };
-
-    // Appends the lanes' candidates (mask4: which of a lane's four elements) in
-    // index order: lane-major, element-minor.  Nearly every call finds a few lanes
-    // with one candidate each: one ballot, one 8-byte LDS store.  Lanes with
-    // several candidates (about one call in ten has one) take the branch that
-    // counts them level by level and stores the rest in a loop.
-    auto append = [&](uint32_t mask4, const u4a& a, uint32_t first_idx) {
-        const uint64_t m1 = __ballot(mask4 != 0);
-        if (!m1) return;  // wave-uniform
-        const uint32_t c = __popc(mask4);
-        uint32_t before = lanes_below(m1), total = __popcll(m1);
-        const uint64_t m2 = __ballot(c >= 2);
-        if (m2) {  // wave-uniform
-            before += lanes_below(m2);
-            total += __popcll(m2);
-            const uint64_t m3 = __ballot(c >= 3);
-            if (m3) {
-                const uint64_t m4 = __ballot(c >= 4);
-                before += lanes_below(m3) + lanes_below(m4);
-                total += __popcll(m3) + __popcll(m4);
-            }
-        }
-        if (dense) return;
-        total = (uint32_t)__builtin_amdgcn_readfirstlane((int)total);
-        if (staged + total > (uint32_t)kRegSlots) {
-            // the region goes dense: its earlier candidates were stored as zeros where
-            // they reached the predicted threshold; put those values back
-            dense = 1u;
-            if ((uint32_t)lane < staged && (stage[wave][lane][1] & 0x7FFFFFFFu) >= that_key)
-                bucket_residual(g, bk, b)[stage[wave][lane][0]] = u2f(stage[wave][lane][1]);
-            return;
-        }
-        if (mask4) {
-            uint32_t pos = staged + before;
-            const uint32_t q = (uint32_t)__ffs((int)mask4) - 1u;
-            slots[pos] = u2a{first_idx + q, pick(a, q)};
-            uint32_t rest = mask4 & (mask4 - 1u);
-            while (rest) {
-                const uint32_t q2 = (uint32_t)__ffs((int)rest) - 1u;
-                slots[++pos] = u2a{first_idx + q2, pick(a, q2)};
-                rest &= rest - 1u;
-            }
-        }
-        staged = (uint32_t)__builtin_amdgcn_readfirstlane((int)(staged + total));
-    };
-
-#pragma unroll
-    for (int round = 0; round < ROUNDS; round++) {
-        if (round + 1 < ROUNDS) issue(round + 1);
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t vi = (uint32_t)(round * U + u) * kWave + lane;
-            u4a a = {0u, 0u, 0u, 0u}, z = {0u, 0u, 0u, 0u};
-            uint32_t mask4 = 0;
-            if (vi < nfull) {
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const float adj = u2f(gv[round][u][q]) + u2f(rv[round][u][q]);
-                    a[q] = f2u(adj);
-                    z[q] = key_of(adj) >= that_key ? 0u : a[q];
-                    mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
-                }
-            }
-            append(mask4, a, (uint32_t)w0 + vi * 4);  // may turn the region dense
-            if (vi < nfull) __builtin_nontemporal_store(dense ? a : z, (u4u4*)(rp + vi * 4));
-        }
-    }
-    // the bucket's last partial vector (bucket length not a multiple of 4) lies in its last region
-    if (len & 3) {
-        u4a a = {0u, 0u, 0u, 0u};
-        uint32_t mask4 = 0;
-        if (lane == 0) {
-            for (uint32_t q = 0; q < (len & 3); q++) {
-                const float adj = gp[nfull * 4 + q] + rp[nfull * 4 + q];
-                a[q] = f2u(adj);
-                mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
-            }
-        }
-        append(mask4, a, (uint32_t)w0 + nfull * 4);
-        if (lane == 0) {
-            for (uint32_t q = 0; q < (len & 3); q++)
-                rp[nfull * 4 + q] = (!dense && (a[q] & 0x7FFFFFFFu) >= that_key) ? 0.0f : u2f(a[q]);
-        }
-    }
-    const uint32_t region = (uint32_t)(w0 / kRegion);
-    if (!dense && (uint32_t)lane < staged) {
-        const u2a e = slots[lane];
-        *(u2a*)(w.list + (((uint64_t)b * g.regions + region) * kRegSlots + lane) * 2) = e;
-    }
-    if (lane == 0) w.reg_cnt[(uint64_t)b * g.regions + region] = dense ? kDense : staged;
-}
-
-// ================================ fused tail ======================================
-// Everything after the streaming pass in one launch: window histogram, threshold
-// bin, exact threshold, tie-break, payload offsets and the payload itself.  The
-// kNSub blocks that work on one bucket meet at two barriers (the histogram is
-// complete; the threshold bin's candidates and the blocks' certain-pick counts
-// are published); nothing else crosses blocks.  Each wavefront owns a contiguous
-// run of regions and keeps their slots in registers across the phases, so the
-// candidate lists are read from memory once.
-//
-// Barrier: a per-bucket arrival counter in the state words (zero at kernel
-// start).  A block's 64 partners are the blocks next to it in dispatch order, so
-// they are resident or about to be; the wait is bounded all the same: a block
-// that waits longer than `limit_ticks` of the 100 MHz wall clock records
-// S_TIMEOUT and leaves, and the call's result for that bucket is then invalid
-// (mccl_hip_topk_path_report returns an error).
-
-constexpr int kTailRegs = 14;  // regions per wavefront whose slots stay in registers
-
+// ---- what blocks of one launch use to talk to each other ----------------------------------
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -958,18 +551,377 @@ __device__ __forceinline__ bool bucket_barrier(uint32_t* counter, uint32_t parti
     return *flag != 0;
 }
 
-// Dense regions (more candidates than slots) are rare.  Every sweep of the tail
-// kernel handles them in a compact loop of its own after the unrolled sweep over
-// the wavefront's register-held regions, so the common path stays small.
-// Calls f(index, bits, in_range) for every element of dense region r, 64 elements
-// per step, every lane of the wavefront taking part in every step; the loads of
-// 16 steps are in flight together and parked in LDS, so the code stays a loop.
-template <class F>
-__device__ __forceinline__ void dense_walk(const float* rp, uint64_t bn, uint32_t r, uint32_t* buf /* 1024 words of LDS per wavefront */,
-                                           F&& f) {
+
+// ================================ single-pass path ==================================
+// Two launches.
+//
+// k_topk_stream - blocks of the 1D grid, in dispatch order:
+//   sample blocks   one per bucket, the first blocks of the grid.  8192 evenly spread
+//                   elements of grad + residual -> the candidate window [lo, hi) and the
+//                   predicted threshold; the block clears the bucket's counters and then
+//                   publishes the call's epoch number in S_READY.
+//   then, segment by segment (segment s = the tiles of bucket s, then the bin blocks of
+//   bucket s - 1; the bin blocks of the last bucket close the grid):
+//   streaming blocks one per 4096-element tile, in address order.  A wavefront loads its
+//                   1024 elements, waits until the bucket's S_READY shows the epoch, stores
+//                   residual <- grad + residual (0.0f at or above the predicted threshold)
+//                   and stages its candidates (key >= lo) in LDS in index order; the block
+//                   writes them to the tile's slots and counts itself into its group of
+//                   tiles (at most 64 groups per bucket).
+//   bin blocks      64 per bucket.  Block g waits until group g's tiles are finished (when it
+//                   is dispatched - one bucket later - they are, except in the last bucket),
+//                   counts the group's candidates per coarse window bin (64 bins), publishes
+//                   the counts and copies the candidates, binned, to the bucket's per-bin
+//                   lists.  It waits for nothing else.
+// k_topk_select - 64 blocks per bucket; nothing crosses blocks any more: every block
+//                   redundantly finds the bin that holds the k-th largest key (from the
+//                   groups' counts), the exact threshold and the tie rule (from that bin's
+//                   list) and the number of picks in the groups before its own, then writes
+//                   its group's picks, in index order, at that offset of the payload and
+//                   repairs the residual where the predicted threshold and the true one
+//                   disagree.  A failed selection (threshold outside the window, a bin list
+//                   overflow) hands the bucket to the exact selection, run by the bucket's 64
+//                   blocks together through counter barriers; the launch covers at most 16
+//                   buckets, so that all its blocks are resident at the same time.
+//
+// Progress in k_topk_stream.  The hardware deals the blocks of a grid to the XCDs round-robin
+// and every XCD dispatches its share in grid order.  A streaming block waits only for its
+// bucket's sample block, which precedes every streaming block in the grid.  A bin block waits
+// only for streaming blocks that precede it in the grid.  Nothing waits for a later block.
+// (Variants in which blocks of the streaming launch also performed the selection were built
+// and measured: with the streaming block that finishes a group last going on as the group's
+// emitter, the slowest XCD collects every emitter, slows down further and jams; with
+// dedicated selection blocks in the grid nothing jams, but every dependent memory round trip
+// of the selection takes 5 to 8 microseconds while the stream is in flight, the blocks live
+// 50 to 100 microseconds each, and the stream loses a quarter of its block slots to them.)
+// All waits are bounded all the same (`limit_ticks`): a block that gives up sets S_TIMEOUT,
+// overwrites the bucket's payload header with kPoisonK and leaves; k_topk_select leaves such
+// a bucket alone.
+//
+// Everything that crosses blocks inside a launch is written and read with agent-scope
+// accesses (the XCDs' L2 caches are not coherent for plain ones), and a writer waits for
+// its stores' acknowledgements before it signals.
+
+constexpr int kFRegion = 1024;                // elements one wavefront streams
+constexpr int kFWaves = kBlock / kWave;       // 4
+constexpr int kFTile = kFRegion * kFWaves;    // elements per streaming block
+constexpr int kFVecs = kFRegion / (kWave * 4);  // 16-byte vectors per lane and array: all issued at once
+constexpr int kTileSlots = 128;               // candidate slots per tile
+constexpr int kCoarse = 64;                   // coarse window bins; the last one holds keys >= hi
+constexpr int kGroups = 64;                   // at most this many groups of tiles per bucket
+constexpr int kCntStride = 64;                // words between two groups' arrival counters: 256 bytes, so that the
+                                              // arrivals of a bucket's tiles spread over memory channels
+constexpr int kHeld = 7;                      // tiles per wavefront whose slots a bin / select block keeps in registers
+constexpr int kFSample = 8192;                // sampled elements per bucket
+constexpr int kSelBuckets = 16;               // buckets per k_topk_select launch: 1024 blocks, all resident
+constexpr uint32_t kPoisonK = 0xFFFFFFFFu;    // payload header of a bucket whose selection was abandoned
+constexpr uint32_t kGaveUp = 0xFFFFFFFEu;     // a wavefront's count: its wait for the sample timed out
+static_assert(kFVecs == 4, "the streaming role is written for four vectors per lane");
+
+__device__ __forceinline__ uint64_t ld_agent64(const uint64_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent64(uint64_t* p, uint64_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 16-byte streaming store written through to memory (agent scope): a later 4-byte
+// repair of the same line by a block on another XCD must not be overwritten by a
+// delayed write-back of this one.  A store of more than 8 bytes reads its data
+// registers over the following cycles: the compiler keeps the next vector
+// instruction from overwriting them for stores it emits itself, not for this one,
+// hence the wait states inside the statement.
+__device__ __forceinline__ void store_through(float* p, u4a v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 2" ::"v"(p), "v"(v) : "memory");
+}
+
+// The window of a bucket, one 16-byte store and one 16-byte load: the four words change together.
+__device__ __forceinline__ void store16_agent(uint32_t* p, u4a v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(p), "v"(v) : "memory");
+}
+// (waits for every earlier load of the wavefront as well: they complete in order)
+__device__ __forceinline__ u4a load16_agent(const uint32_t* p) {
+    u4a v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    return v;
+}
+// Coarse bins are 2^shift keys wide: the smallest shift that fits [lo, hi) into kCoarse - 1 bins.
+__device__ __forceinline__ uint32_t window_shift(uint32_t lo, uint32_t hi) {
+    uint32_t shift = 0;
+    while (((hi - lo) >> shift) >= (uint32_t)(kCoarse - 1)) shift++;
+    return shift;
+}
+
+struct FusedGeo {       // per-bucket tiling, derived the same way by every block
+    uint64_t bn;        // elements
+    uint32_t k;
+    uint32_t ntiles;    // streaming tiles
+    uint32_t tpg;       // tiles per group
+    uint32_t ng;        // groups
+};
+__device__ __forceinline__ FusedGeo fused_geo(const Geometry& g, BucketsArg bk, uint32_t b) {
+    FusedGeo f;
+    f.bn = bucket_count(g, bk, b);
+    f.k = bucket_k(g, bk, b);
+    f.ntiles = (uint32_t)((f.bn + kFTile - 1) / kFTile);
+    f.tpg = (f.ntiles + kGroups - 1) / kGroups;
+    f.ng = (f.ntiles + f.tpg - 1) / f.tpg;
+    return f;
+}
+
+// Coarse window bin of a candidate key (key >= lo).
+__device__ __forceinline__ uint32_t coarse_bin(uint32_t key, uint32_t lo, uint32_t hi, uint32_t shift) {
+    return key >= hi ? (uint32_t)(kCoarse - 1) : (key - lo) >> shift;
+}
+
+// Waits until *p == want.  Called by a whole wavefront or a single thread; false when the wait timed out.
+// Every poll is a memory transaction on one address (agent-scope loads are not cached):
+// few pollers and a pause between polls, or the channel that holds the word becomes the
+// bottleneck of every stream that crosses it.
+__device__ __forceinline__ bool wait_word(const uint32_t* p, uint32_t want, uint64_t limit_ticks) {
+    uint64_t t0 = 0;
+    uint32_t polls = 0;
+    while ((uint32_t)__builtin_amdgcn_readfirstlane((int)ld_agent(p)) != want) {
+        __builtin_amdgcn_s_sleep(16);
+        if ((++polls & 63u) == 0) {
+            const uint64_t now = (uint64_t)wall_clock64();
+            if (t0 == 0) t0 = now;
+            else if (now - t0 > limit_ticks) return false;
+        }
+    }
+    asm volatile("" ::: "memory");
+    return true;
+}
+
+// Waits until the bucket's window is published (S_READY == epoch); called by a whole wavefront
+// or a single thread.  win[3] = 0 when the wait timed out.
+__device__ __forceinline__ u4a wait_window(const uint32_t* st, uint32_t epoch, uint64_t limit_ticks) {
+    uint64_t t0 = 0;
+    uint32_t polls = 0;
+    for (;;) {
+        u4a v = load16_agent(st + S_LO_KEY);
+        if ((uint32_t)__builtin_amdgcn_readfirstlane((int)v[3]) == epoch) {
+            v[3] = 1u;
+            return v;
+        }
+        __builtin_amdgcn_s_sleep(16);
+        if ((++polls & 63u) == 0) {
+            const uint64_t now = (uint64_t)wall_clock64();
+            if (t0 == 0) t0 = now;
+            else if (now - t0 > limit_ticks) {
+                v[3] = 0u;
+                return v;
+            }
+        }
+    }
+}
+
+struct StreamLds {
+    union {
+        struct {  // sample block
+            uint32_t lh[3][kBinsR] __attribute__((aligned(16)));
+            uint32_t wsum[3][kBlock / kWave];
+            uint32_t res[3][2];
+        } s;
+        struct {  // streaming block
+            uint64_t stage[kFWaves][kWave];  // a wavefront's candidates, (bits << 32) | index, in index order
+            uint32_t wcnt[kFWaves];
+            uint32_t win[4];                 // the bucket's window as wavefront 0 read it: lo, hi, predicted threshold, ready
+        } a;
+        struct {  // bin block
+            uint32_t dbuf[kFWaves][16 * kWave];  // dense_tile_walk's staging area, one per wavefront
+            uint32_t cnt[kCoarse];
+            uint32_t base[kCoarse];
+            uint32_t win[4];
+        } e;
+    };
+};
+struct SelectLds {
+    uint32_t lh[kBins0];                 // radix rounds, tie-break, exact fallback
+    // dense_tile_walk's staging area, one per wavefront; the threshold bin's list in between
+    uint32_t dbuf[kFWaves][16 * kWave] __attribute__((aligned(8)));
+    uint32_t part[kFWaves][kCoarse];
+    uint32_t rcnt[kFWaves][kHeld];
+    uint32_t wtot[kFWaves];
+    uint32_t scratch[kBlock / kWave + 2];
+    uint32_t flag;
+};
+
+// ---- sample ------------------------------------------------------------------------
+// For NR ranks at once: the bin in which a top-down scan of histogram h[z] reaches rank[z],
+// and how many of the rank's elements fall inside that bin.  Thread t owns the PER bins below
+// BINS - PER t (16-byte LDS reads).  res[z] = {bin, left}; bin = BINS when the histogram holds
+// fewer than rank[z] elements or rank[z] == 0.  Called by all threads of the block.
+template <int BINS, int NR>
+__device__ __forceinline__ void sample_pick(const uint32_t* const (&h)[NR], const uint32_t (&rank)[NR],
+                                            uint32_t (*wsum)[kBlock / kWave], uint32_t (*res)[2]) {
+    constexpr int PER = BINS / kBlock;
+    static_assert(PER % 4 == 0, "16-byte LDS reads");
     const int lane = threadIdx.x & (kWave - 1);
-    const uint64_t e0 = (uint64_t)r * kRegion;
-    const uint64_t e1 = e0 + kRegion < bn ? e0 + kRegion : bn;
+    const int wave = threadIdx.x / kWave;
+    uint32_t c[NR][PER], sum[NR], inc[NR];  // c[z][j]: bin BINS - 1 - PER t - j
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        const u4a* row = (const u4a*)&h[z][BINS - PER * (threadIdx.x + 1)];
+        sum[z] = 0;
+#pragma unroll
+        for (int v4 = 0; v4 < PER / 4; v4++) {
+            const u4a x = row[PER / 4 - 1 - v4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                c[z][v4 * 4 + q] = x[3 - q];
+                sum[z] += x[3 - q];
+            }
+        }
+        inc[z] = wave_inclusive_scan(sum[z]);
+        if (lane == kWave - 1) wsum[z][wave] = inc[z];
+    }
+    if (threadIdx.x < NR) { res[threadIdx.x][0] = BINS; res[threadIdx.x][1] = 0; }
+    __syncthreads();
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        uint32_t above = inc[z] - sum[z];
+#pragma unroll
+        for (int i = 0; i < kBlock / kWave; i++)
+            if (i < wave) above += wsum[z][i];
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            if (above < rank[z] && rank[z] <= above + c[z][j]) {
+                res[z][0] = (uint32_t)(BINS - 1 - PER * (int)threadIdx.x - j);
+                res[z][1] = rank[z] - above;
+            }
+            above += c[z][j];
+        }
+    }
+    __syncthreads();
+}
+
+// Radix-selects (11 + 10 key bits) three ranks of the sample, whose keys stay in registers:
+// upper and lower end of the candidate window, 6 sigma of the sampling noise away from the
+// expected rank of the k-th largest key, and the predicted threshold.  Clears what the
+// launches accumulate into, then publishes the window and the epoch with one store.
+__device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, const Workspace& w, uint32_t b,
+                                             uint32_t epoch, StreamLds& L) {
+    const FusedGeo fg = fused_geo(g, bk, b);
+    const uint64_t bn = fg.bn;
+    const float* gp = bucket_grad(g, bk, b);
+    const float* rp = bucket_residual(g, bk, b);
+    const uint64_t nvec = bn / 4;
+    constexpr int SV = kFSample / 4;     // sampled vectors
+    constexpr int PV = SV / kBlock;      // vectors per thread; their 4 * PV keys stay in registers
+    // sampled in runs of 8 vectors (one 128-byte line per array), runs evenly spread
+    const uint32_t nsv = nvec < (uint64_t)SV ? (uint32_t)(nvec & ~7ull) : (uint32_t)SV;
+    const uint64_t stride = nsv ? (nvec / (nsv / 8)) : 8;  // vectors between run starts (>= 8)
+    u4a gv[PV], rv[PV];
+#pragma unroll
+    for (int j = 0; j < PV; j++) {
+        const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
+        const uint32_t ii = i < nsv ? i : 0;
+        const uint64_t v = (uint64_t)(ii >> 3) * stride + (ii & 7);
+        gv[j] = nsv ? *(const u4u4*)(gp + v * 4) : u4a{0u, 0u, 0u, 0u};
+        rv[j] = nsv ? *(const u4u4*)(rp + v * 4) : u4a{0u, 0u, 0u, 0u};
+    }
+    // while the loads are under way: clear what the launches accumulate into (the
+    // acknowledgements are back long before the window is published)
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    if (threadIdx.x < kGroups) st_agent(w.grp_cnt + ((uint64_t)b * kGroups + threadIdx.x) * kCntStride, 0u);
+    if (threadIdx.x < kCoarse) st_agent(w.bin_fill + (uint64_t)b * kCoarse + threadIdx.x, 0u);
+    if (threadIdx.x == 0) {
+        st_agent(st + S_OK, 0u);
+        st_agent(st + S_TIMEOUT, 0u);
+        st_agent(st + S_BARF, 0u); st_agent(st + S_BARF + 1, 0u); st_agent(st + S_BARF + 2, 0u); st_agent(st + S_BARF + 3, 0u);
+    }
+    uint32_t* const h0 = &L.s.lh[0][0];  // round 0 uses 2048 bins: lh[0] and lh[1] are adjacent
+    {
+        const u4a z = {0u, 0u, 0u, 0u};
+        for (int i = threadIdx.x; i < 3 * kBinsR / 4; i += kBlock) ((u4a*)h0)[i] = z;
+    }
+    uint32_t key[PV][4];
+#pragma unroll
+    for (int j = 0; j < PV; j++) {
+        // an element past the sample gets the key 0xFFFFFFFF, which no histogram counts
+        const bool have = (uint32_t)j * kBlock + threadIdx.x < nsv;
+#pragma unroll
+        for (int q = 0; q < 4; q++) key[j][q] = have ? key_of(u2f(gv[j][q]) + u2f(rv[j][q])) : 0xFFFFFFFFu;
+    }
+    const uint32_t S = nsv * 4;
+    const float ks = (float)fg.k * (float)S / (float)bn;
+    const float margin = 6.0f * sqrtf(ks) + 16.0f;
+    // ranks: 0 upper end of the window, 1 lower end, 2 the predicted threshold itself
+    constexpr int NR = 3;
+    uint32_t rank[NR];
+    rank[0] = ks - margin >= 1.0f ? (uint32_t)(ks - margin) : 0u;  // 0: no upper end
+    rank[1] = (uint32_t)(ks + margin) + 1u;                       // > S: no lower end
+    rank[2] = ks >= 1.0f ? (uint32_t)ks : 1u;
+    const bool active[NR] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S, rank[2] <= S};
+    uint32_t prefix[NR];
+    __syncthreads();
+    // round 0: key[30:20], one histogram for all ranks
+#pragma unroll
+    for (int j = 0; j < PV; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (key[j][q] != 0xFFFFFFFFu) atomicAdd(&h0[key[j][q] >> 20], 1u);
+    __syncthreads();
+    {
+        const uint32_t* const hs[NR] = {h0, h0, h0};
+        const uint32_t want[NR] = {active[0] ? rank[0] : 0u, active[1] ? rank[1] : 0u, active[2] ? rank[2] : 0u};
+        sample_pick<kBins0, NR>(hs, want, L.s.wsum, L.s.res);
+    }
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        prefix[z] = L.s.res[z][0] << 20;
+        rank[z] = L.s.res[z][1];
+    }
+    __syncthreads();
+    // round 1: key[19:10] among the keys that share a rank's first digit
+    {
+        const u4a z = {0u, 0u, 0u, 0u};
+        for (int i = threadIdx.x; i < 3 * kBinsR / 4; i += kBlock) ((u4a*)h0)[i] = z;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PV; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t kq = key[j][q];
+#pragma unroll
+            for (int z = 0; z < NR; z++)
+                if (active[z] && (kq >> 20) == (prefix[z] >> 20)) atomicAdd(&L.s.lh[z][(kq >> 10) & (kBinsR - 1)], 1u);
+        }
+    __syncthreads();
+    {
+        const uint32_t* const hs[NR] = {L.s.lh[0], L.s.lh[1], L.s.lh[2]};
+        const uint32_t want[NR] = {active[0] ? rank[0] : 0u, active[1] ? rank[1] : 0u, active[2] ? rank[2] : 0u};
+        sample_pick<kBinsR, NR>(hs, want, L.s.wsum, L.s.res);
+    }
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int z = 0; z < NR; z++) prefix[z] |= (L.s.res[z][0] & (uint32_t)(kBinsR - 1)) << 10;
+        const uint32_t lo = active[1] ? prefix[1] : 0u;
+        uint32_t hi = active[0] ? (prefix[0] | 0x3FFu) : 0x7FFFFFFFu;  // upper end of the window: rounded up
+        if (hi < lo) hi = lo;
+        // predicted threshold: middle of its 1024-key cell; never below lo: every pre-zeroed
+        // element must be a listed candidate
+        uint32_t that = active[2] ? (prefix[2] | 0x200u) : 0x7FFFFFFFu;
+        if (that < lo) that = lo;
+        // every store above must have arrived before the window is published
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        store16_agent(st + S_LO_KEY, u4a{lo, hi, that, epoch});
+    }
+    // off the critical path: the histograms of the exact selection, should the select launch need it
+    for (int i = threadIdx.x; i < kHistWords; i += kBlock) w.hist[(uint64_t)b * kHistWords + i] = 0u;
+}
+
+// ---- a dense tile's elements ---------------------------------------------------------
+// Calls f(index, bits, in_range) for every element of tile t of the bucket, 64 elements per
+// step, every lane of the wavefront taking part in every step; the loads of 16 steps are in
+// flight together and parked in LDS, so the code stays a loop.  AGENT: the residual was
+// written by other blocks of the same launch.
+template <bool AGENT, class F>
+__device__ __forceinline__ void dense_tile_walk(const float* rp, uint64_t bn, uint32_t t, uint32_t* buf, F&& f) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint64_t e0 = (uint64_t)t * kFTile;
+    const uint64_t e1 = e0 + kFTile < bn ? e0 + kFTile : bn;
     constexpr int B = 16;
 #pragma unroll 1
     for (uint64_t base = e0; base < e1; base += (uint64_t)B * kWave) {
@@ -977,7 +929,8 @@ __device__ __forceinline__ void dense_walk(const float* rp, uint64_t bn, uint32_
 #pragma unroll
         for (int j = 0; j < B; j++) {
             const uint64_t i = base + (uint64_t)j * kWave + lane;
-            v[j] = i < e1 ? f2u(rp[i]) : 0u;
+            if constexpr (AGENT) v[j] = i < e1 ? ld_agent((const uint32_t*)rp + i) : 0u;
+            else v[j] = i < e1 ? f2u(rp[i]) : 0u;
         }
 #pragma unroll
         for (int j = 0; j < B; j++) buf[j * kWave + lane] = v[j];  // a lane reads back only what it wrote
@@ -989,11 +942,359 @@ __device__ __forceinline__ void dense_walk(const float* rp, uint64_t bn, uint32_
     }
 }
 
-// The need-th smallest index among list2's entries with key == T (ties at the
-// threshold go to the lower index): radix select over the index, 11 + 11 + 10 bits.
-// Called by all threads of the block.
-__device__ __forceinline__ uint32_t resolve_ties(const uint32_t* l2, uint32_t count2, uint32_t T, uint32_t need,
-                                              uint32_t* lh /* kBins0 words */, uint32_t* scratch) {
+// ---- a group's tiles as a bin block / select block sees them ------------------------------
+// The slots of up to kHeld tiles per wavefront stay in registers, the rest (buckets of more
+// than 64 * 4 * kHeld tiles) are re-read from memory on every sweep.  AGENT: the slots were
+// written by other blocks of the same launch (agent-scope loads), else by an earlier launch.
+template <bool AGENT>
+struct GroupTiles {
+    const uint32_t* tcnt;
+    const uint64_t* slots;
+    uint32_t t0;        // the group's first tile
+    uint32_t wt0, wt1;  // this wavefront's tiles: a contiguous quarter of the group's
+    int lane;
+    bool more;          // wave-uniform: dense tiles, or tiles past the register window
+    uint32_t cnt[kHeld];            // candidates in the tile's slots, or kDense (wave-uniform)
+    uint64_t e0[kHeld], e1[kHeld];  // slot `lane` and slot `64 + lane`
+
+    static __device__ __forceinline__ uint32_t ld32(const uint32_t* p) {
+        if constexpr (AGENT) return ld_agent(p);
+        else return *p;
+    }
+    static __device__ __forceinline__ uint64_t ld64(const uint64_t* p) {
+        if constexpr (AGENT) return ld_agent64(p);
+        else return *p;
+    }
+    // every load issued at once
+    __device__ __forceinline__ void load(const Geometry& g, const Workspace& w, uint32_t b, uint32_t grp,
+                                         const FusedGeo& fg) {
+        constexpr int NW = kBlock / kWave;
+        lane = threadIdx.x & (kWave - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+        tcnt = w.tile_cnt + (uint64_t)b * g.ftiles;
+        slots = w.slots + (uint64_t)b * g.ftiles * kTileSlots;
+        t0 = grp * fg.tpg;
+        const uint32_t t1 = t0 + fg.tpg < fg.ntiles ? t0 + fg.tpg : fg.ntiles;
+        const uint32_t pw = (t1 - t0 + NW - 1) / NW;
+        wt0 = t0 + wave * pw < t1 ? t0 + wave * pw : t1;
+        wt1 = wt0 + pw < t1 ? wt0 + pw : t1;
+#pragma unroll
+        for (int h = 0; h < kHeld; h++) {
+            const uint32_t t = wt0 + h < wt1 ? wt0 + h : t0;  // stays inside the bucket's arrays
+            cnt[h] = (uint32_t)__builtin_amdgcn_readfirstlane((int)ld32(tcnt + t));
+            e0[h] = ld64(slots + (uint64_t)t * kTileSlots + lane);  // slots past the count: ignored by the sweeps
+            e1[h] = ld64(slots + (uint64_t)t * kTileSlots + kWave + lane);
+        }
+        bool any_dense = false;
+#pragma unroll
+        for (int h = 0; h < kHeld; h++) any_dense |= wt0 + h < wt1 && cnt[h] == kDense;
+        more = any_dense || wt1 > wt0 + kHeld;
+    }
+    // nd(h, t, cnt, e0, e1) for every ordinary tile (h < kHeld: register-held, else ~0u), dn(h, t)
+    // for every dense one.  Order: register-held ordinary tiles first, then the dense ones and
+    // those past the register window, in index order.
+    template <class ND, class DN>
+    __device__ __forceinline__ void sweep(ND&& nd, DN&& dn) const {
+#pragma unroll
+        for (int h = 0; h < kHeld; h++)
+            if (wt0 + h < wt1 && cnt[h] != kDense) nd((uint32_t)h, wt0 + h, cnt[h], e0[h], e1[h]);
+        if (more) {
+#pragma unroll 1
+            for (uint32_t t = wt0; t < wt1; t++) {
+                const uint32_t h = t - wt0 < (uint32_t)kHeld ? t - wt0 : ~0u;
+                const uint32_t c = (uint32_t)__builtin_amdgcn_readfirstlane((int)ld32(tcnt + t));
+                if (c == kDense) {
+                    dn(h, t);
+                } else if (h == ~0u) {
+                    const uint64_t a0 = ld64(slots + (uint64_t)t * kTileSlots + lane);
+                    const uint64_t a1 = ld64(slots + (uint64_t)t * kTileSlots + kWave + lane);
+                    nd(h, t, c, a0, a1);
+                }
+            }
+        }
+    }
+};
+__device__ __forceinline__ uint32_t key64(uint64_t e) { return (uint32_t)(e >> 32) & 0x7FFFFFFFu; }
+
+__device__ __forceinline__ void fused_give_up(const Workspace& w, uint32_t* st, uint32_t* out) {
+    if (threadIdx.x == 0) {
+        st_agent(st + S_TIMEOUT, 1u);
+        if (w.status) st_agent((uint32_t*)w.status, (uint32_t)MCCL_HIP_ERR_TIMEOUT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        st_agent(out, kPoisonK);
+    }
+}
+
+// ---- bin block -----------------------------------------------------------------------------
+__device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, const Workspace& w, uint32_t b,
+                                          uint32_t grp, const FusedGeo& fg, uint32_t epoch, uint64_t limit_ticks,
+                                          StreamLds& L) {
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    // the group's tiles are finished: all its streaming blocks have arrived
+    {
+        const uint32_t tg0 = grp * fg.tpg;
+        const uint32_t in_group = (tg0 + fg.tpg < fg.ntiles ? tg0 + fg.tpg : fg.ntiles) - tg0;
+        // the counter is only meaningful once the sample block has cleared it
+        if (threadIdx.x == 0) {
+            u4a wn = wait_window(st, epoch, limit_ticks);
+            if (wn[3] && !wait_word(w.grp_cnt + ((uint64_t)b * kGroups + grp) * kCntStride, in_group, limit_ticks)) wn[3] = 0u;
+            L.e.win[0] = wn[0]; L.e.win[1] = wn[1]; L.e.win[2] = wn[2]; L.e.win[3] = wn[3];
+        }
+        __syncthreads();
+        if (!L.e.win[3]) {
+            fused_give_up(w, st, bucket_wire(g, bk, b));
+            return;
+        }
+    }
+    const uint32_t lo = L.e.win[0], hi = L.e.win[1], shift = window_shift(L.e.win[0], L.e.win[1]);
+    const uint64_t bn = fg.bn;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const float* rp = bucket_residual(g, bk, b);
+    GroupTiles<true> G;
+    G.load(g, w, b, grp, fg);
+    // candidates per coarse bin
+    if (threadIdx.x < kCoarse) L.e.cnt[threadIdx.x] = 0;
+    __syncthreads();
+    G.sweep([&](uint32_t, uint32_t, uint32_t cnt, uint64_t a0, uint64_t a1) {
+                if ((uint32_t)lane < cnt) atomicAdd(&L.e.cnt[coarse_bin(key64(a0), lo, hi, shift)], 1u);
+                if ((uint32_t)(kWave + lane) < cnt) atomicAdd(&L.e.cnt[coarse_bin(key64(a1), lo, hi, shift)], 1u);
+            },
+            [&](uint32_t, uint32_t t) {
+                dense_tile_walk<true>(rp, bn, t, L.e.dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
+                    const uint32_t key = v & 0x7FFFFFFFu;
+                    const bool cand = in && key >= lo;
+                    wave_hist_add(L.e.cnt, cand, cand ? coarse_bin(key, lo, hi, shift) : 0u);
+                });
+            });
+    __syncthreads();
+    if (threadIdx.x < kCoarse) {
+        const uint32_t c = L.e.cnt[threadIdx.x];
+        w.ghist[((uint64_t)b * kGroups + grp) * kCoarse + threadIdx.x] = c;
+        // the top bin (keys >= hi) holds picks for certain as long as the window holds: no list
+        L.e.base[threadIdx.x] = (c && threadIdx.x < kCoarse - 1)
+            ? __hip_atomic_fetch_add(w.bin_fill + (uint64_t)b * kCoarse + threadIdx.x, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+            : 0u;
+    }
+    __syncthreads();
+    // binned copies (read by the next launch: plain stores)
+    uint64_t* bl = w.blist + (uint64_t)b * (kCoarse - 1) * g.lcapb;
+    auto put = [&](bool valid, uint32_t cb, uint64_t e) {
+        if (valid && cb < (uint32_t)(kCoarse - 1)) {
+            const uint32_t pos = atomicAdd(&L.e.base[cb], 1u);
+            if (pos < g.lcapb) bl[(uint64_t)cb * g.lcapb + pos] = e;
+        }
+    };
+    G.sweep([&](uint32_t, uint32_t, uint32_t cnt, uint64_t a0, uint64_t a1) {
+                put((uint32_t)lane < cnt, coarse_bin(key64(a0), lo, hi, shift), a0);
+                put((uint32_t)(kWave + lane) < cnt, coarse_bin(key64(a1), lo, hi, shift), a1);
+            },
+            [&](uint32_t, uint32_t t) {
+                dense_tile_walk<true>(rp, bn, t, L.e.dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
+                    const uint32_t key = v & 0x7FFFFFFFu;
+                    const bool cand = in && key >= lo;
+                    put(cand, cand ? coarse_bin(key, lo, hi, shift) : 0u, (uint64_t)i | ((uint64_t)v << 32));
+                });
+            });
+}
+
+// ---- the streaming launch ------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, Workspace w, uint32_t epoch,
+                                                        uint32_t first_wave, uint64_t limit_ticks) {
+    const BucketsArg bk = buckets_arg();
+    __shared__ StreamLds L;
+    if (blockIdx.x < g.nbuckets) {
+        fused_sample(bk, g, w, blockIdx.x, epoch, L);
+        return;
+    }
+    // segment s of the grid: the tiles of bucket s, then the bin blocks of bucket s - 1 (whose
+    // tiles are finished or about to be by then: a bin block that is dispatched early only
+    // polls); after the last segment the bin blocks of the last bucket
+    const uint32_t per = g.ftiles + kGroups;
+    const uint32_t j = blockIdx.x - g.nbuckets;
+    uint32_t b = j / per, t = j - b * per;
+    bool emit = false;
+    if (b >= g.nbuckets) {
+        t = j - g.nbuckets * per;
+        b = g.nbuckets - 1;
+        emit = true;
+    } else if (t >= g.ftiles) {
+        if (b == 0) return;
+        t -= g.ftiles;
+        b -= 1;
+        emit = true;
+    }
+    const FusedGeo fg = fused_geo(g, bk, b);
+    if (emit) {
+        if (t < fg.ng) fused_bin(bk, g, w, b, t, fg, epoch, limit_ticks, L);
+        return;
+    }
+    if (t >= fg.ntiles) return;
+    // The blocks that start together with the sample blocks would bury the samples' few loads under
+    // 40 MB of their own and then wait for the samples all the same: they hold back for two
+    // microseconds, and the memory system is busy with their loads while the samples are evaluated.
+    if (blockIdx.x < first_wave) __builtin_amdgcn_s_sleep(80);
+    const uint64_t bn = fg.bn;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const uint64_t w0 = (uint64_t)t * kFTile + (uint64_t)wave * kFRegion;  // first element of this wave's region
+    const bool live = w0 < bn;                                             // wave-uniform
+    float* const rbase = bucket_residual(g, bk, b);
+    const float* gp = bucket_grad(g, bk, b) + w0;
+    float* rp = rbase + w0;
+    const uint32_t len = live ? (uint32_t)((bn - w0) < (uint64_t)kFRegion ? (bn - w0) : (uint64_t)kFRegion) : 0u;
+    const uint32_t nfull = len / 4;  // full vectors in this region
+    u4a gv[kFVecs], rv[kFVecs];
+#pragma unroll
+    for (int u = 0; u < kFVecs; u++) {
+        const uint32_t vi = (uint32_t)u * kWave + lane;
+        if (vi < nfull) {
+            gv[u] = __builtin_nontemporal_load((const u4u4*)(gp + vi * 4));
+            rv[u] = __builtin_nontemporal_load((const u4u4*)(rp + vi * 4));
+        }
+    }
+    uint32_t* st = w.state + (uint64_t)b * kStateWords;
+    uint32_t* out = bucket_wire(g, bk, b);
+    // the window of this bucket: wait for its sample block (one wavefront polls for the block)
+    if (wave == 0) {
+        const u4a wn = wait_window(st, epoch, limit_ticks);
+        if (lane == 0) { L.a.win[0] = wn[0]; L.a.win[1] = wn[1]; L.a.win[2] = wn[2]; L.a.win[3] = wn[3]; }
+    }
+    __syncthreads();
+    const bool ready = L.a.win[3] != 0;
+    const uint32_t lo_key = L.a.win[0], that_key = L.a.win[2];
+    // both the same in every lane, and kept in scalar registers by saying so at every update
+    uint32_t staged = 0;  // candidates of the region so far
+    uint32_t dense = 0;   // 1: more candidates than slots
+    uint64_t* const slots = L.a.stage[wave];
+    auto lanes_below = [&](uint64_t m) {
+        return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+    };
+    auto pick = [](const u4a& a, uint32_t q) {
+        uint32_t v = a[0];
+        v = q == 1 ? a[1] : v;
+        v = q == 2 ? a[2] : v;
+        return q == 3 ? a[3] : v;
+    };
+    // Puts back the region's staged candidates that were stored as zeros.
+    auto restore_staged = [&]() {
+        if ((uint32_t)lane < staged) {
+            const uint64_t e = slots[lane];
+            if (((uint32_t)(e >> 32) & 0x7FFFFFFFu) >= that_key) st_agent((uint32_t*)rbase + (uint32_t)e, (uint32_t)(e >> 32));
+        }
+    };
+    // Appends the lanes' candidates (mask4: which of a lane's four elements) in index
+    // order: lane-major, element-minor.  Nearly every call finds a few lanes with one
+    // candidate each: one ballot, one 8-byte LDS store.
+    auto append = [&](uint32_t mask4, const u4a& a, uint32_t first_idx) {
+        const uint64_t m1 = __ballot(mask4 != 0);
+        if (!m1) return;  // wave-uniform
+        const uint32_t c = __popc(mask4);
+        uint32_t before = lanes_below(m1), total = __popcll(m1);
+        const uint64_t m2 = __ballot(c >= 2);
+        if (m2) {  // wave-uniform
+            before += lanes_below(m2);
+            total += __popcll(m2);
+            const uint64_t m3 = __ballot(c >= 3);
+            if (m3) {
+                const uint64_t m4 = __ballot(c >= 4);
+                before += lanes_below(m3) + lanes_below(m4);
+                total += __popcll(m3) + __popcll(m4);
+            }
+        }
+        if (dense) return;
+        total = (uint32_t)__builtin_amdgcn_readfirstlane((int)total);
+        if (staged + total > (uint32_t)kWave) {
+            // the region goes dense: its earlier candidates were stored as zeros where
+            // they reached the predicted threshold; put those values back
+            dense = 1u;
+            restore_staged();
+            return;
+        }
+        if (mask4) {
+            uint32_t pos = staged + before;
+            const uint32_t q = (uint32_t)__ffs((int)mask4) - 1u;
+            slots[pos] = (uint64_t)(first_idx + q) | ((uint64_t)pick(a, q) << 32);
+            uint32_t rest = mask4 & (mask4 - 1u);
+            while (rest) {
+                const uint32_t q2 = (uint32_t)__ffs((int)rest) - 1u;
+                slots[++pos] = (uint64_t)(first_idx + q2) | ((uint64_t)pick(a, q2) << 32);
+                rest &= rest - 1u;
+            }
+        }
+        staged = (uint32_t)__builtin_amdgcn_readfirstlane((int)(staged + total));
+    };
+    if (ready) {
+#pragma unroll
+        for (int u = 0; u < kFVecs; u++) {
+            const uint32_t vi = (uint32_t)u * kWave + lane;
+            u4a a = {0u, 0u, 0u, 0u}, z = {0u, 0u, 0u, 0u};
+            uint32_t mask4 = 0;
+            if (vi < nfull) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float adj = u2f(gv[u][q]) + u2f(rv[u][q]);
+                    a[q] = f2u(adj);
+                    z[q] = key_of(adj) >= that_key ? 0u : a[q];
+                    mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
+                }
+            }
+            append(mask4, a, (uint32_t)w0 + vi * 4);  // may turn the region dense
+            if (vi < nfull) store_through(rp + vi * 4, dense ? a : z);
+        }
+        // the bucket's last partial vector (bucket length not a multiple of 4) lies in its last region
+        if (len & 3) {
+            u4a a = {0u, 0u, 0u, 0u};
+            uint32_t mask4 = 0;
+            if (lane == 0) {
+                for (uint32_t q = 0; q < (len & 3); q++) {
+                    const float adj = gp[nfull * 4 + q] + rp[nfull * 4 + q];
+                    a[q] = f2u(adj);
+                    mask4 |= (key_of(adj) >= lo_key ? 1u : 0u) << q;
+                }
+            }
+            append(mask4, a, (uint32_t)w0 + nfull * 4);
+            if (lane == 0) {
+                for (uint32_t q = 0; q < (len & 3); q++)
+                    st_agent((uint32_t*)rp + nfull * 4 + q, (!dense && (a[q] & 0x7FFFFFFFu) >= that_key) ? 0u : a[q]);
+            }
+        }
+    }
+    // ---- the tile's candidates, in index order, to its slots ------------------------------
+    if (lane == 0) L.a.wcnt[wave] = !ready ? kGaveUp : (dense ? kDense : staged);
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+    bool tile_dense = false, gave_up = false;
+#pragma unroll
+    for (int i = 0; i < kFWaves; i++) {
+        const uint32_t c = L.a.wcnt[i];
+        gave_up |= c == kGaveUp;
+        tile_dense |= c == kDense;
+        if (i < wave) before += c;
+        total += c;
+    }
+    if (gave_up) {  // a wavefront never saw the sample arrive: the bucket's result is invalid
+        fused_give_up(w, st, out);
+        return;     // without counting the tile: the bucket's bin blocks give up as well
+    }
+    tile_dense |= total > (uint32_t)kTileSlots;
+    if (tile_dense) {
+        if (!dense) restore_staged();  // a tile is dense as a whole: its residual holds plain sums
+    } else if ((uint32_t)lane < staged) {
+        st_agent64(w.slots + ((uint64_t)b * g.ftiles + t) * kTileSlots + before + lane, slots[lane]);
+    }
+    if (threadIdx.x == 0) st_agent(w.tile_cnt + (uint64_t)b * g.ftiles + t, tile_dense ? kDense : total);
+    // ---- the block counts itself into its group once all its stores have arrived ----------
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(w.grp_cnt + ((uint64_t)b * kGroups + t / fg.tpg) * kCntStride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The need-th smallest index among the list's entries with key == T: radix select over
+// the index, 11 + 11 + 10 bits.  Called by all threads of the block.
+__device__ __forceinline__ uint32_t resolve_ties64(const uint64_t* l2, uint32_t count2, uint32_t T, uint32_t need,
+                                                   uint32_t* lh /* kBins0 words */, uint32_t* scratch) {
     uint32_t iwant = need, iprefix = 0;
     const int shifts[3] = {21, 10, 0};
     const int widths[3] = {11, 11, 10};
@@ -1003,14 +1304,14 @@ __device__ __forceinline__ uint32_t resolve_ties(const uint32_t* l2, uint32_t co
         __syncthreads();
         const int hs = shifts[r] + widths[r];
         for (uint32_t i = threadIdx.x; i < count2; i += kBlock) {
-            const uint32_t idx = ld_agent(&l2[2 * (uint64_t)i]), key = ld_agent(&l2[2 * (uint64_t)i + 1]);
+            const uint64_t e = l2[i];
+            const uint32_t idx = (uint32_t)e, key = (uint32_t)(e >> 32) & 0x7FFFFFFFu;
             const bool match = hs >= 32 ? true : ((idx >> hs) == (iprefix >> hs));
             // bins stored reversed, so that pick_bin's top-down scan runs over ascending indices
             if (key == T && match) atomicAdd(&lh[(bins - 1) - ((idx >> shifts[r]) & (bins - 1))], 1u);
         }
         __syncthreads();
         uint32_t left;
-        // a 1024-bin round leaves the upper half of the 2048 bins empty: one scan serves both widths
         const uint32_t rb = pick_bin<kBins0, kBlock>(lh, iwant, 0, &left, scratch);
         iprefix |= ((uint32_t)(bins - 1) - (rb - (uint32_t)(kBins0 - bins))) << shifts[r];
         iwant = left;
@@ -1018,51 +1319,31 @@ __device__ __forceinline__ uint32_t resolve_ties(const uint32_t* l2, uint32_t co
     return iprefix;
 }
 
-// The exact selection of one bucket by the kNSub blocks that work on it: the
-// fallback for a bucket whose window could not finish the selection (too few
-// candidates, threshold outside the window, a threshold bin with more keys than
-// list2 holds).  No extra launch; every block of the bucket enters it together.
-//   1  each block puts back, in its own regions, what the streaming pass stored as 0.0f
-//   2  three radix rounds over the key (11 + 10 + 10 bits): a block histograms its
-//      own slice of the bucket in LDS and adds it to the bucket's histogram; after
-//      a barrier every block scans that histogram and gets the same digit
-//   3  a block counts the keys above and at the threshold in its slice; after a
-//      barrier every block knows how many picks precede its slice
-//   4  a block writes its slice's picks in index order and zeroes them
-// A block only ever reads the residual range it restored itself, so the residual
-// needs no exchange between blocks.  lh: kBins0 words, scratch: kBlock / kWave + 2
-// words, flag: one word of LDS.  Returns false when a barrier wait timed out;
-// *T_out receives the exact threshold key.
-__device__ __forceinline__ bool bucket_exact_group(BucketsArg bk, const Geometry& g, const Workspace& w,
-                                                   uint32_t b, uint32_t s, const Window& wn, uint32_t* lh,
-                                                   uint32_t* scratch, uint32_t* flag, uint64_t limit_ticks,
-                                                   uint32_t* T_out) {
+
+// The exact selection of one bucket by its select blocks together (same algorithm as the exact
+// path: three radix rounds over the key, then an ordered emit), each on its own group's
+// element range; four barriers.  Returns false when a barrier wait timed out.
+__device__ __forceinline__ bool select_exact_group(BucketsArg bk, const Geometry& g, const Workspace& w, uint32_t b,
+                                                   uint32_t grp, const FusedGeo& fg, uint32_t that_key,
+                                                   const GroupTiles<false>& G, SelectLds& L, uint64_t limit_ticks) {
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const uint64_t bn = bucket_count(g, bk, b);
+    const uint64_t bn = fg.bn;
     float* rp = bucket_residual(g, bk, b);
-    uint32_t r0, r1;
-    block_regions(g, bk, b, s, &r0, &r1);
-    const uint64_t e0 = (uint64_t)r0 * kRegion;
-    const uint64_t e1 = (uint64_t)r1 * kRegion < bn ? (uint64_t)r1 * kRegion : bn;
-    // 1: this block's regions
-    {
-        const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
-        const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-        for (uint32_t slot = r0 * kRegSlots + threadIdx.x; slot < r1 * kRegSlots; slot += kBlock) {
-            const uint32_t cnt = rc[slot / kRegSlots];
-            if (cnt == kDense || (slot % kRegSlots) >= cnt) continue;
-            const uint32_t idx = lb[2 * (uint64_t)slot], bitsv = lb[2 * (uint64_t)slot + 1];
-            if ((bitsv & 0x7FFFFFFFu) >= wn.that) rp[idx] = u2f(bitsv);
-        }
-        __syncthreads();
-    }
-    // 2: radix select.  Every wavefront walks a contiguous quarter of the block's slice,
-    // 64 elements per step with the loads of eight steps in flight; f(i, bits, valid) is
-    // called by all lanes of the wavefront for every step.
-    constexpr int NW = kBlock / kWave;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const uint64_t below = (1ull << lane) - 1ull;
+    const uint64_t e0 = (uint64_t)grp * fg.tpg * kFTile;
+    const uint64_t e1r = e0 + (uint64_t)fg.tpg * kFTile;
+    const uint64_t e1 = e1r < bn ? e1r : bn;
+    // 1: put back what the streaming blocks stored as 0.0f in this group's tiles
+    G.sweep([&](uint32_t, uint32_t, uint32_t cnt, uint64_t a0, uint64_t a1) {
+                if ((uint32_t)lane < cnt && key64(a0) >= that_key) rp[(uint32_t)a0] = u2f((uint32_t)(a0 >> 32));
+                if ((uint32_t)(kWave + lane) < cnt && key64(a1) >= that_key) rp[(uint32_t)a1] = u2f((uint32_t)(a1 >> 32));
+            },
+            [&](uint32_t, uint32_t) {});
+    __syncthreads();  // a block only ever reads the range it restored itself: plain accesses
+    // 2: radix select; every wavefront walks a contiguous quarter of the group's range
+    constexpr int NW = kBlock / kWave;
     const uint64_t quarter = ((e1 - e0 + NW - 1) / NW + kWave - 1) / kWave * kWave;
     const uint64_t ws0 = e0 + (uint64_t)wave * quarter < e1 ? e0 + (uint64_t)wave * quarter : e1;
     const uint64_t ws1 = ws0 + quarter < e1 ? ws0 + quarter : e1;
@@ -1083,8 +1364,9 @@ __device__ __forceinline__ bool bucket_exact_group(BucketsArg bk, const Geometry
             }
         }
     };
-    uint32_t* gh = w.hist + (uint64_t)b * kHistWords;  // zero at kernel start
-    uint32_t prefix = 0, remaining = bucket_k(g, bk, b);
+    uint32_t* lh = L.lh;
+    uint32_t* gh = w.hist + (uint64_t)b * kHistWords;  // cleared by the bucket's sample block
+    uint32_t prefix = 0, remaining = fg.k;
 #pragma unroll 1
     for (int round = 0; round < 3; round++) {
         const int bins = round == 0 ? kBins0 : kBinsR;
@@ -1102,17 +1384,17 @@ __device__ __forceinline__ bool bucket_exact_group(BucketsArg bk, const Geometry
             const uint32_t c = lh[i];
             if (c) __hip_atomic_fetch_add(&ghr[i], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (!bucket_barrier(st + S_BARF + round, kNSub, flag, limit_ticks)) return false;
+        if (!bucket_barrier(st + S_BARF + round, fg.ng, &L.flag, limit_ticks)) return false;
         for (int i = threadIdx.x; i < bins; i += kBlock) lh[i] = ld_agent(&ghr[i]);
         __syncthreads();
         uint32_t left, bin;
-        if (round == 0) bin = pick_bin<kBins0, kBlock>(lh, remaining, 0, &left, scratch);
-        else bin = pick_bin<kBinsR, kBlock>(lh, remaining, 0, &left, scratch);
+        if (round == 0) bin = pick_bin<kBins0, kBlock>(lh, remaining, 0, &left, L.scratch);
+        else bin = pick_bin<kBinsR, kBlock>(lh, remaining, 0, &left, L.scratch);
         prefix |= bin << shift;
         remaining = left;
     }
     const uint32_t T = prefix, need = remaining;
-    // 3: keys above and at the threshold per wavefront range, per block, and in the slices before
+    // 3: keys above and at the threshold per wavefront range, per group, and in the groups before
     uint32_t gt_w = 0, eq_w = 0;  // wave-uniform
     walk([&](uint64_t, uint32_t v, bool valid) {
         const uint32_t key = v & 0x7FFFFFFFu;
@@ -1131,24 +1413,22 @@ __device__ __forceinline__ bool bucket_exact_group(BucketsArg bk, const Geometry
         eq_blk += wsum[NW + i];
     }
     if (threadIdx.x == 0) {
-        st_agent(&w.blk_above[(uint64_t)b * kNSub + s], gt_blk);
-        st_agent(&w.blk_eq[(uint64_t)b * kNSub + s], eq_blk);
+        st_agent(&w.blk_above[(uint64_t)b * kGroups + grp], gt_blk);
+        st_agent(&w.blk_eq[(uint64_t)b * kGroups + grp], eq_blk);
     }
-    if (!bucket_barrier(st + S_BARF + 3, kNSub, flag, limit_ticks)) return false;
+    if (!bucket_barrier(st + S_BARF + 3, fg.ng, &L.flag, limit_ticks)) return false;
     {
-        static_assert(kNSub <= kBlock, "one thread per block of the bucket");
-        const uint32_t vg = threadIdx.x < s ? ld_agent(&w.blk_above[(uint64_t)b * kNSub + threadIdx.x]) : 0u;
-        const uint32_t ve = threadIdx.x < s ? ld_agent(&w.blk_eq[(uint64_t)b * kNSub + threadIdx.x]) : 0u;
+        static_assert(kGroups <= kBlock, "one thread per group of the bucket");
+        const uint32_t vg = threadIdx.x < grp ? ld_agent(&w.blk_above[(uint64_t)b * kGroups + threadIdx.x]) : 0u;
+        const uint32_t ve = threadIdx.x < grp ? ld_agent(&w.blk_eq[(uint64_t)b * kGroups + threadIdx.x]) : 0u;
         uint32_t gt_before, eq_before;
-        block_exclusive_scan(vg, scratch, &gt_before);
-        block_exclusive_scan(ve, scratch, &eq_before);
+        block_exclusive_scan(vg, L.scratch, &gt_before);
+        block_exclusive_scan(ve, L.scratch, &eq_before);
         gt_run += gt_before;
         eq_run += eq_before;
     }
-    // 4: this wavefront's picks, in index order: an element lands at (keys above T before it)
-    // + min(keys equal to T before it, need); ties are taken while fewer than need came before
+    // 4: this wavefront's picks, in index order
     uint32_t* out = bucket_wire(g, bk, b);
-    if (s == 0 && threadIdx.x == 0) out[0] = bucket_k(g, bk, b);
     walk([&](uint64_t i, uint32_t v, bool valid) {
         const uint32_t key = v & 0x7FFFFFFFu;
         const bool is_gt = valid && key > T, is_eq = valid && key == T;
@@ -1164,207 +1444,112 @@ __device__ __forceinline__ bool bucket_exact_group(BucketsArg bk, const Geometry
         gt_run += (uint32_t)__popcll(mg);
         eq_run += (uint32_t)__popcll(me);
     });
-    *T_out = T;
+    if (grp == 0 && threadIdx.x == 0) {
+        st[S_T] = T;
+        st[S_NEED] = need;
+    }
     return true;
 }
 
-__global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Workspace w, uint64_t limit_ticks) {
+
+// ---- the select launch ----------------------------------------------------------------------
+// blockIdx.x = group, blockIdx.y = bucket - first_bucket.  Everything the streaming launch
+// left behind is read with plain loads; only the exact fallback talks across blocks.
+__global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, Workspace w, uint32_t first_bucket,
+                                                           uint64_t limit_ticks) {
     const BucketsArg bk = buckets_arg();
+    __shared__ SelectLds L;
     constexpr int NW = kBlock / kWave;
-    __shared__ uint32_t lh[kBins0];
-    __shared__ uint32_t scratch[NW + 2];
-    __shared__ uint32_t sh_a[NW], sh_b[NW], sh_x[2];
-    __shared__ uint32_t rcnt[NW][kTailRegs];  // phase 4: picks per register-held region
-    __shared__ uint32_t dbuf[NW][16 * kWave];  // dense_walk's staging area, one per wavefront
-    const uint32_t b = blockIdx.y, s = blockIdx.x;
+    const uint32_t b = first_bucket + blockIdx.y, grp = blockIdx.x;
+    const FusedGeo fg = fused_geo(g, bk, b);
+    if (grp >= fg.ng) return;
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
-    const Window wn = load_window(st);
-    const uint32_t lo = wn.lo, hi = wn.hi, shift = wn.shift, that_key = wn.that;
-    const uint32_t k = bucket_k(g, bk, b);
-    const uint64_t bn = bucket_count(g, bk, b);
-    uint32_t r0, r1;
-    block_regions(g, bk, b, s, &r0, &r1);
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
-    const uint64_t below = (1ull << lane) - 1ull;
-    // this wavefront's regions: a contiguous quarter of the block's
-    const uint32_t pw = (r1 - r0 + NW - 1) / NW;
-    const uint32_t wr0 = r0 + wave * pw < r1 ? r0 + wave * pw : r1;
-    const uint32_t wr1 = wr0 + pw < r1 ? wr0 + pw : r1;
-    const uint32_t* rc = w.reg_cnt + (uint64_t)b * g.regions;
-    const uint32_t* lb = w.list + (uint64_t)b * g.regions * kRegSlots * 2;
-    float* rp = bucket_residual(g, bk, b);
-    uint32_t* hw = w.hist_w + (uint64_t)b * kWinBins;
-    uint32_t* l2 = w.list2 + (uint64_t)b * g.lcap2 * 2;
-    uint32_t* above_of = w.blk_above + (uint64_t)b * kNSub;
     uint32_t* out = bucket_wire(g, bk, b);
+    if (st[S_TIMEOUT]) return;  // the streaming launch gave the bucket up: its payload header says so
+    if (grp == 0 && threadIdx.x == 0) st[S_READY] = 0u;  // a replay of a captured launch carries the same epoch
+    GroupTiles<false> G;
+    G.load(g, w, b, grp, fg);
+    const uint32_t lo = st[S_LO_KEY], that_key = st[S_THAT], shift = window_shift(lo, st[S_HI_KEY]);
+    const uint32_t k = fg.k;
+    const uint64_t bn = fg.bn;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const uint64_t below = (1ull << lane) - 1ull;
+    float* rp = bucket_residual(g, bk, b);
 
-    // ---- slots of the first kTailRegs regions into registers, every load issued at once
-    uint32_t ccnt[kTailRegs], cidx[kTailRegs], cbits[kTailRegs];
-#pragma unroll
-    for (int q = 0; q < kTailRegs; q++) {
-        const uint32_t r = wr0 + q < wr1 ? wr0 + q : (wr1 > wr0 ? wr1 - 1 : 0);  // stays inside the bucket's lists
-        ccnt[q] = rc[r];
-        const u2a e = *(const u2a*)(lb + 2 * ((uint64_t)r * kRegSlots + lane));  // slots past the count: ignored below
-        cidx[q] = e[0];
-        cbits[q] = e[1];
-    }
-    bool any_dense = false;  // wave-uniform: one of the register-held regions is dense
-#pragma unroll
-    for (int q = 0; q < kTailRegs; q++) any_dense |= wr0 + q < wr1 && ccnt[q] == kDense;
-
-    // A sweep = nd(q, r, cnt, idx, bits) for every ordinary region (q < kTailRegs: register-held,
-    // else ~0u), dn(q, r) for every dense one.  Order: register-held ordinary regions first, then
-    // the dense ones and those past the register window, in index order.
-    const bool more = any_dense || wr1 > wr0 + kTailRegs;  // wave-uniform
-    auto sweep = [&](auto&& nd, auto&& dn) {
-#pragma unroll
-        for (int q = 0; q < kTailRegs; q++)
-            if (wr0 + q < wr1 && ccnt[q] != kDense) nd((uint32_t)q, wr0 + q, ccnt[q], cidx[q], cbits[q]);
-        if (more) {
-#pragma unroll 1
-            for (uint32_t r = wr0; r < wr1; r++) {
-                const uint32_t q = r - wr0 < (uint32_t)kTailRegs ? r - wr0 : ~0u;
-                const uint32_t cnt = rc[r];
-                if (cnt == kDense) {
-                    dn(q, r);
-                } else if (q == ~0u) {
-                    const u2a e = *(const u2a*)(lb + 2 * ((uint64_t)r * kRegSlots + lane));
-                    nd(q, r, cnt, e[0], e[1]);
-                }
-            }
-        }
-    };
-    // Reasons to hand the bucket to the exact selection are collected in `failed`
-    // (block-uniform, and the same in every block of the bucket); the one call sits
-    // at the end of the kernel.
     bool failed = false;
-
-    // ---- phase 1: window histogram -------------------------------------------------
-    // (A window that does not fit the histogram - only possible when the state words hold
-    // foreign contents - skips the work but not the barrier: a block that reaches the end
-    // of the kernel may rewrite the window, so every block must have read it by then.)
-    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = 0;
-    __syncthreads();
-    if (wn.sound)
-    sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t, uint32_t bitsv) {
-              if ((uint32_t)lane < cnt) atomicAdd(&lh[window_bin(bitsv & 0x7FFFFFFFu, lo, hi, shift)], 1u);
-          },
-          [&](uint32_t, uint32_t r) {
-              dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
-                  const uint32_t key = v & 0x7FFFFFFFu;
-                  const bool cand = in && key >= lo;
-                  wave_hist_add(lh, cand, cand ? window_bin(key, lo, hi, shift) : 0u);
-              });
-          });
-    __syncthreads();
-    for (int i = threadIdx.x; i < kWinBins; i += kBlock) {
-        const uint32_t c = lh[i];
-        if (c) __hip_atomic_fetch_add(&hw[i], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (!bucket_barrier(st + S_BAR1, kNSub, &sh_x[0], limit_ticks)) {
-        if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
-        return;
-    }
-
     do {
-    if (!wn.sound) {
-        failed = true;
-        break;
-    }
-    // ---- phase 2: threshold bin; certain picks per block; the bin's candidates to list2
-    for (int i = threadIdx.x; i < kWinBins; i += kBlock) lh[i] = ld_agent(&hw[i]);
-    __syncthreads();
-    uint32_t need;
-    const uint32_t jstar = pick_bin<kWinBins, kBlock>(lh, k, 0, &need, scratch);
-    if (jstar >= (uint32_t)(kWinBins - 1)) {  // fewer than k candidates, or the threshold lies above the window
-        failed = true;
-        break;
-    }
-    uint32_t w_above = 0, w_hits = 0;
-    sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t, uint32_t bitsv) {
-              const bool valid = (uint32_t)lane < cnt;
-              const uint32_t bin = valid ? window_bin(bitsv & 0x7FFFFFFFu, lo, hi, shift) : 0u;
-              w_above += (uint32_t)__popcll(__ballot(valid && bin > jstar));
-              w_hits += (uint32_t)__popcll(__ballot(valid && bin == jstar));
-          },
-          [&](uint32_t, uint32_t r) {
-              dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
-                  const uint32_t key = v & 0x7FFFFFFFu;
-                  const bool cand = in && key >= lo;
-                  const uint32_t bin = cand ? window_bin(key, lo, hi, shift) : 0u;
-                  w_above += (uint32_t)__popcll(__ballot(cand && bin > jstar));
-                  w_hits += (uint32_t)__popcll(__ballot(cand && bin == jstar));
-              });
-          });
-    if (lane == 0) { sh_a[wave] = w_above; sh_b[wave] = w_hits; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t ta = 0, th = 0;
+    // ---- 3: threshold bin from the groups' counts -------------------------------------------
+    // thread (wave, lane): bin `lane` of groups [16 wave, 16 wave + 16)
+    constexpr int GPW = kGroups / NW;
+    uint32_t gh[GPW];
+    uint32_t mine = 0;
 #pragma unroll
-        for (int i = 0; i < NW; i++) { ta += sh_a[i]; th += sh_b[i]; }
-        st_agent(&above_of[s], ta);
-        sh_x[1] = th ? __hip_atomic_fetch_add(st + S_N2, th, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    for (int i = 0; i < GPW; i++) {
+        const uint32_t gi = (uint32_t)(wave * GPW + i);
+        gh[i] = gi < fg.ng ? w.ghist[((uint64_t)b * kGroups + gi) * kCoarse + lane] : 0u;
+        mine += gh[i];
     }
+    L.part[wave][lane] = mine;
     __syncthreads();
-    if (w_hits) {  // wave-uniform; list2's order does not matter
-        uint32_t pos = sh_x[1];
-        for (int i = 0; i < wave; i++) pos += sh_b[i];
-        auto put = [&](bool hit, uint32_t idx, uint32_t key) {
-            const uint64_t m = __ballot(hit);
-            if (hit) {
-                const uint32_t p = pos + (uint32_t)__popcll(m & below);
-                if (p < g.lcap2) {
-                    st_agent(&l2[2 * (uint64_t)p], idx);
-                    st_agent(&l2[2 * (uint64_t)p + 1], key);
-                }
-            }
-            pos += (uint32_t)__popcll(m);
-        };
-        sweep([&](uint32_t, uint32_t, uint32_t cnt, uint32_t idx, uint32_t bitsv) {
-                  const uint32_t key = bitsv & 0x7FFFFFFFu;
-                  put((uint32_t)lane < cnt && window_bin(key, lo, hi, shift) == jstar, idx, key);
-              },
-              [&](uint32_t, uint32_t r) {
-                  dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
-                      const uint32_t key = v & 0x7FFFFFFFu;
-                      put(in && key >= lo && window_bin(key, lo, hi, shift) == jstar, i, key);
-                  });
-              });
+    // scanned from the top bin downwards: lane l looks at bin 63 - l
+    uint32_t totr = 0;
+#pragma unroll
+    for (int i = 0; i < NW; i++) totr += L.part[i][kCoarse - 1 - lane];
+    const uint32_t inc = wave_inclusive_scan(totr);
+    const uint64_t reach = __ballot(inc >= k);
+    if (!reach) {  // fewer than k candidates
+        failed = true;
+        break;
     }
-    if (!bucket_barrier(st + S_BAR2, kNSub, &sh_x[0], limit_ticks)) {
-        if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
-        return;
+    const int lstar = __ffsll((long long)reach) - 1;
+    const uint32_t jstar = (uint32_t)(kCoarse - 1 - lstar);
+    if (jstar == (uint32_t)(kCoarse - 1)) {  // the threshold lies at or above the window's upper end
+        failed = true;
+        break;
+    }
+    const uint32_t n2 = (uint32_t)__shfl((int)totr, lstar, kWave);          // candidates in the threshold bin
+    const uint32_t above_total = (uint32_t)__shfl((int)inc, lstar, kWave) - n2;
+    const uint32_t need = k - above_total;                                   // picks inside the bin, 1..n2
+    // certain picks (bins above the threshold bin) in the groups before this one
+    uint32_t ab = 0;
+#pragma unroll
+    for (int i = 0; i < GPW; i++)
+        if ((uint32_t)lane > jstar && (uint32_t)(wave * GPW + i) < grp) ab += gh[i];
+    uint32_t above_before;
+    block_exclusive_scan(ab, L.scratch, &above_before);
+    if (n2 > g.lcapb) {  // more keys in the threshold bin than its list holds (heavy ties, clustered values)
+        failed = true;
+        break;
     }
 
-    // ---- phase 3: exact threshold from list2 (every block, redundantly) -----------------
-    // every load of this phase is issued at once: the entries do not wait for their count
-    // (slots past it hold leftovers and are masked below)
-    constexpr int kL2Regs = 4;  // list2 entries per thread kept in registers (1024 per block)
-    uint32_t eidx[kL2Regs], ekey[kL2Regs];
+    // ---- 4: exact threshold from the bin's list ---------------------------------------------
+    const uint64_t* l2 = w.blist + ((uint64_t)b * (kCoarse - 1) + jstar) * g.lcapb;
+    // the first 2048 entries are parked in LDS (the dense walks' staging area is idle until the emit)
+    constexpr uint32_t kL2Cached = kFWaves * 16 * kWave / 2;
+    uint64_t* const lcache = (uint64_t*)&L.dbuf[0][0];
+    {
+        constexpr int PER = kL2Cached / kBlock;
+        uint64_t ent[PER];
 #pragma unroll
-    for (int j = 0; j < kL2Regs; j++) {
-        const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
-        eidx[j] = i < g.lcap2 ? ld_agent(&l2[2 * (uint64_t)i]) : 0u;
-        ekey[j] = i < g.lcap2 ? ld_agent(&l2[2 * (uint64_t)i + 1]) : 0u;
-    }
-    const uint32_t above_mine = threadIdx.x < (uint32_t)kNSub ? ld_agent(&above_of[threadIdx.x]) : 0u;
-    const uint32_t count2 = ld_agent(st + S_N2);
-    if (count2 > g.lcap2) {  // more keys in the threshold bin than list2 holds (heavy ties)
-        failed = true;
-        break;
+        for (int j = 0; j < PER; j++) {
+            const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
+            ent[j] = i < n2 ? l2[i] : 0ull;
+        }
+#pragma unroll
+        for (int j = 0; j < PER; j++) lcache[(uint32_t)j * kBlock + threadIdx.x] = ent[j];  // a thread reads back only what it wrote
     }
     auto for_list2 = [&](auto&& body) {
-#pragma unroll
-        for (int j = 0; j < kL2Regs; j++)
-            if ((uint32_t)j * kBlock + threadIdx.x < count2) body(eidx[j], ekey[j]);
 #pragma unroll 1
-        for (uint32_t i = kL2Regs * kBlock + threadIdx.x; i < count2; i += kBlock)
-            body(ld_agent(&l2[2 * (uint64_t)i]), ld_agent(&l2[2 * (uint64_t)i + 1]));
+        for (uint32_t i = threadIdx.x; i < n2; i += kBlock) {
+            const uint64_t e = i < kL2Cached ? lcache[i] : l2[i];
+            body((uint32_t)e, key64(e));
+        }
     };
+    uint32_t* lh = L.lh;
     const uint32_t bin_lo = lo + (jstar << shift);  // smallest key of the threshold bin
     uint32_t vprefix = 0, want = need;              // key - bin_lo: up to 30 bits, selected as 10 + 10 + 10
-    // a window bin spans 2^shift keys: rounds whose digits lie wholly above that are skipped
+    // a bin spans 2^shift keys: rounds whose digits lie wholly above that are skipped
     const int first_round = shift <= 10 ? 2 : (shift <= 20 ? 1 : 0);
 #pragma unroll 1
     for (int r = first_round; r < 3; r++) {
@@ -1378,62 +1563,78 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Wo
         });
         __syncthreads();
         uint32_t left;
-        const uint32_t bin = pick_bin<kBinsR, kBlock>(lh, want, 0, &left, scratch);
+        const uint32_t bin = pick_bin<kBinsR, kBlock>(lh, want, 0, &left, L.scratch);
+        if (bin >= (uint32_t)kBinsR) {  // the list holds fewer matching keys than the counts promised
+            failed = true;
+            break;
+        }
         vprefix |= bin << sh;
         want = left;
     }
+    if (failed) break;
     const uint32_t T = bin_lo + vprefix;
     const uint32_t need2 = want;
     const uint32_t ties = lh[vprefix & (kBinsR - 1)];
     __syncthreads();
     // when only some keys equal to T are taken, they are the need2 lowest indices
-    const uint32_t istar = ties != need2 ? resolve_ties(l2, count2, T, need2, lh, scratch) : 0xFFFFFFFFu;
+    const uint32_t istar = ties != need2 ? resolve_ties64(l2, n2, T, need2, lh, L.scratch) : 0xFFFFFFFFu;
     auto is_pick = [&](bool valid, uint32_t key, uint32_t idx) {
         return valid && (key > T || (key == T && idx <= istar));
     };
-    // picks before this block's first element: the earlier blocks' certain picks and the
-    // threshold bin's picks at lower indices
+    // the threshold bin's picks at indices below this group's first element
     uint32_t mine_before = 0, mine_all = 0;
-    const uint64_t first_elem = (uint64_t)r0 * kRegion;
+    const uint64_t first_elem = (uint64_t)G.t0 * kFTile;
     for_list2([&](uint32_t idx, uint32_t key) {
         if (is_pick(true, key, idx)) {
             mine_all++;
             mine_before += (uint64_t)idx < first_elem ? 1u : 0u;
         }
     });
-    uint32_t l2_before, l2_total, above_before, above_total;
-    block_exclusive_scan(mine_before, scratch, &l2_before);
-    block_exclusive_scan(mine_all, scratch, &l2_total);
-    block_exclusive_scan(threadIdx.x < s ? above_mine : 0u, scratch, &above_before);
-    block_exclusive_scan(above_mine, scratch, &above_total);
+    uint32_t l2_before, l2_total;
+    block_exclusive_scan(mine_before, L.scratch, &l2_before);
+    block_exclusive_scan(mine_all, L.scratch, &l2_total);
     if (above_total + l2_total != k) {  // cannot happen with consistent lists
         failed = true;
         break;
     }
 
-    // ---- phase 4: payload, in index order -----------------------------------------------
-    // picks per region first: the register-held regions' into rcnt, the others' into a total
+    // ---- 5: payload, in index order -----------------------------------------------------------
+    // picks per tile first: the register-held tiles' into rcnt, the others' into the total
     uint32_t w_total = 0;
-    sweep([&](uint32_t q, uint32_t, uint32_t cnt, uint32_t idx, uint32_t bitsv) {
-              const uint32_t c = (uint32_t)__popcll(__ballot(is_pick((uint32_t)lane < cnt, bitsv & 0x7FFFFFFFu, idx)));
-              if (q != ~0u) rcnt[wave][q] = c;
+    G.sweep([&](uint32_t h, uint32_t, uint32_t cnt, uint64_t a0, uint64_t a1) {
+              const uint32_t c = (uint32_t)__popcll(__ballot(is_pick((uint32_t)lane < cnt, key64(a0), (uint32_t)a0))) +
+                                 (uint32_t)__popcll(__ballot(is_pick((uint32_t)(kWave + lane) < cnt, key64(a1), (uint32_t)a1)));
+              if (h != ~0u) L.rcnt[wave][h] = c;
               w_total += c;
           },
-          [&](uint32_t q, uint32_t r) {
+          [&](uint32_t h, uint32_t t) {
               uint32_t c = 0;
-              dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
-                  c += (uint32_t)__popcll(__ballot(is_pick(in, v & 0x7FFFFFFFu, i)));
+              dense_tile_walk<false>(rp, bn, t, L.dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
+                  c += (uint32_t)__popcll(__ballot(is_pick(in && (v & 0x7FFFFFFFu) >= lo, v & 0x7FFFFFFFu, i)));
               });
-              if (q != ~0u) rcnt[wave][q] = c;
+              if (h != ~0u) L.rcnt[wave][h] = c;
               w_total += c;
           });
-    if (lane == 0) sh_a[wave] = w_total;
+    if (lane == 0) L.wtot[wave] = w_total;
     __syncthreads();
     uint32_t wave_off = above_before + l2_before;
-    for (int i = 0; i < wave; i++) wave_off += sh_a[i];
-    auto emit_dense = [&](uint32_t r, uint32_t pos) {
-        dense_walk(rp, bn, r, dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
-            const bool pick = is_pick(in, v & 0x7FFFFFFFu, i);
+    for (int i = 0; i < wave; i++) wave_off += L.wtot[i];
+    auto emit_half = [&](bool valid, uint64_t e, uint32_t pos) {
+        const uint32_t key = key64(e), idx = (uint32_t)e, bitsv = (uint32_t)(e >> 32);
+        const bool pick = is_pick(valid, key, idx);
+        const uint64_t m = __ballot(pick);
+        if (pick) {
+            const u2a pr = {idx, bitsv};
+            *(u2a4*)(out + 1 + 2 * (uint64_t)(pos + (uint32_t)__popcll(m & below))) = pr;
+        }
+        // the streaming block stored 0.0f for key >= predicted threshold; repair where the prediction was wrong
+        if (valid && pick != (key >= that_key)) rp[idx] = pick ? 0.0f : u2f(bitsv);
+        return pos + (uint32_t)__popcll(m);
+    };
+    auto emit_dense = [&](uint32_t t, uint32_t pos) {
+        // a dense tile's residual holds plain sums (nothing was stored as zero)
+        dense_tile_walk<false>(rp, bn, t, L.dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
+            const bool pick = is_pick(in && (v & 0x7FFFFFFFu) >= lo, v & 0x7FFFFFFFu, i);
             const uint64_t m = __ballot(pick);
             if (pick) {
                 const uint32_t p = pos + (uint32_t)__popcll(m & below);
@@ -1445,80 +1646,64 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_tail(Buckets, Geometry g, Wo
         });
         return pos;
     };
-    auto emit_region = [&](uint32_t cnt, uint32_t idx, uint32_t bitsv, uint32_t pos) {
-        const bool valid = (uint32_t)lane < cnt;
-        const uint32_t key = bitsv & 0x7FFFFFFFu;
-        const bool pick = is_pick(valid, key, idx);
-        const uint64_t m = __ballot(pick);
-        if (pick) {
-            const u2a e = {idx, bitsv};
-            *(u2a4*)(out + 1 + 2 * (uint64_t)(pos + (uint32_t)__popcll(m & below))) = e;
-        }
-        // pass A stored 0.0f for key >= predicted threshold; repair where the prediction was wrong
-        if (valid && pick != (key >= that_key)) rp[idx] = pick ? 0.0f : u2f(bitsv);
-        return pos + (uint32_t)__popcll(m);
-    };
     {
         uint32_t pos = wave_off;
 #pragma unroll
-        for (int q = 0; q < kTailRegs; q++) {
-            if (wr0 + q < wr1) {
-                if (ccnt[q] != kDense) pos = emit_region(ccnt[q], cidx[q], cbits[q], pos);
-                else pos += rcnt[wave][q];  // written out by the loop below
+        for (int h = 0; h < kHeld; h++) {
+            if (G.wt0 + h < G.wt1) {
+                if (G.cnt[h] != kDense) {
+                    pos = emit_half((uint32_t)lane < G.cnt[h], G.e0[h], pos);
+                    pos = emit_half((uint32_t)(kWave + lane) < G.cnt[h], G.e1[h], pos);
+                } else {
+                    pos += L.rcnt[wave][h];  // written out by the loop below
+                }
             }
         }
     }
-    if (more) {
+    if (G.more) {
         uint32_t pos = wave_off;
 #pragma unroll 1
-        for (uint32_t r = wr0; r < wr1; r++) {
-            const uint32_t cnt = rc[r];
+        for (uint32_t t = G.wt0; t < G.wt1; t++) {
+            const uint32_t cnt = (uint32_t)__builtin_amdgcn_readfirstlane((int)G.tcnt[t]);
             if (cnt == kDense) {
-                pos = emit_dense(r, pos);
-            } else if (r - wr0 < (uint32_t)kTailRegs) {
-                pos += rcnt[wave][r - wr0];
+                pos = emit_dense(t, pos);
+            } else if (t - G.wt0 < (uint32_t)kHeld) {
+                pos += L.rcnt[wave][t - G.wt0];
             } else {
-                const u2a e = *(const u2a*)(lb + 2 * ((uint64_t)r * kRegSlots + lane));
-                pos = emit_region(cnt, e[0], e[1], pos);
+                const uint64_t a0 = G.slots[(uint64_t)t * kTileSlots + lane];
+                const uint64_t a1 = G.slots[(uint64_t)t * kTileSlots + kWave + lane];
+                pos = emit_half((uint32_t)lane < cnt, a0, pos);
+                pos = emit_half((uint32_t)(kWave + lane) < cnt, a1, pos);
             }
         }
     }
-    if (s == 0 && threadIdx.x == 0) {
-        out[0] = k;
+    if (grp == 0 && threadIdx.x == 0) {
         st[S_T] = T;
         st[S_NEED] = need2;
         st[S_ISTAR] = istar;
         st[S_OK] = 1u;
-        predict_next_window(st, T);
     }
     } while (false);
     // the exact selection for a bucket the window could not finish (S_OK stays 0)
     if (failed) {
-        uint32_t T;
-        if (!bucket_exact_group(bk, g, w, b, s, wn, lh, scratch, &sh_x[0], limit_ticks, &T)) {
-            if (threadIdx.x == 0) st_agent(st + S_TIMEOUT, 1u);
+        if (!select_exact_group(bk, g, w, b, grp, fg, that_key, G, L, limit_ticks)) {
+            fused_give_up(w, st, out);
             return;
         }
-        if (s == 0 && threadIdx.x == 0) predict_next_window(st, T);
     }
+    if (grp == 0 && threadIdx.x == 0 && !ld_agent(st + S_TIMEOUT)) out[0] = k;
 }
-
-#include "topk_fused.hip.h"
 
 // ================================ host side =======================================
 
 uint64_t align4(uint64_t words) { return (words + 3) & ~uint64_t(3); }
 
 uint64_t zeroed_words(const Geometry& g) {
-    return align4((uint64_t)g.nbuckets * kHistWords) + align4((uint64_t)g.nbuckets * kWinBins) +
-           align4((uint64_t)g.nbuckets * kStateWords);
+    return align4((uint64_t)g.nbuckets * kHistWords) + align4((uint64_t)g.nbuckets * kStateWords);
 }
 
 uint64_t workspace_words(const Geometry& g) {
-    return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) +
-           align4((uint64_t)g.nbuckets * g.regions) +
-           align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2) + align4((uint64_t)g.nbuckets * g.lcap2 * 2) +
-           2 * align4((uint64_t)g.nbuckets * kNSub) +
+    return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) + 2 * align4((uint64_t)g.nbuckets * kGroups) +
            align4((uint64_t)g.nbuckets * g.ftiles) + align4((uint64_t)g.nbuckets * g.ftiles * kTileSlots * 2) +
            align4((uint64_t)g.nbuckets * kGroups * kCntStride) + align4((uint64_t)g.nbuckets * kGroups * kCoarse) +
            align4((uint64_t)g.nbuckets * kCoarse) + align4((uint64_t)g.nbuckets * (kCoarse - 1) * g.lcapb * 2);
@@ -1528,21 +1713,18 @@ Workspace carve(void* base, const Geometry& g) {
     Workspace w;
     uint32_t* p = (uint32_t*)base;
     w.hist = p;        p += align4((uint64_t)g.nbuckets * kHistWords);
-    w.hist_w = p;      p += align4((uint64_t)g.nbuckets * kWinBins);
     w.state = p;       p += align4((uint64_t)g.nbuckets * kStateWords);
     w.tile_gt = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
     w.tile_eq = p;     p += align4((uint64_t)g.nbuckets * g.tiles);
-    w.reg_cnt = p;     p += align4((uint64_t)g.nbuckets * g.regions);
-    w.list = p;        p += align4((uint64_t)g.nbuckets * g.regions * kRegSlots * 2);
-    w.list2 = p;       p += align4((uint64_t)g.nbuckets * g.lcap2 * 2);
-    w.blk_above = p;   p += align4((uint64_t)g.nbuckets * kNSub);
-    w.blk_eq = p;      p += align4((uint64_t)g.nbuckets * kNSub);
+    w.blk_above = p;   p += align4((uint64_t)g.nbuckets * kGroups);
+    w.blk_eq = p;      p += align4((uint64_t)g.nbuckets * kGroups);
     w.tile_cnt = p;    p += align4((uint64_t)g.nbuckets * g.ftiles);
     w.slots = (uint64_t*)p;  p += align4((uint64_t)g.nbuckets * g.ftiles * kTileSlots * 2);
     w.grp_cnt = p;     p += align4((uint64_t)g.nbuckets * kGroups * kCntStride);
     w.ghist = p;       p += align4((uint64_t)g.nbuckets * kGroups * kCoarse);
     w.bin_fill = p;    p += align4((uint64_t)g.nbuckets * kCoarse);
     w.blist = (uint64_t*)p;
+    w.status = nullptr;
     return w;
 }
 
@@ -1558,12 +1740,6 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     g->tiles = (uint32_t)((bucket_elems + kTile - 1) / kTile);
     g->k_full = mccl_hip_topk_k(bucket_elems, ratio);
     g->k_last = mccl_hip_topk_k(n_total - (nb - 1) * bucket_elems, ratio);
-    g->regions = (uint32_t)((bucket_elems + kATile - 1) / kATile) * (kATile / kRegion);
-    // list2 holds the candidates of one window bin (1/256 of about 1.7 k in the expected
-    // case); 2 k + 4096 entries leave room for heavy ties, never more than the bucket
-    uint64_t cap = 2 * (uint64_t)g->k_full + 4096;
-    if (cap > bucket_elems) cap = bucket_elems;
-    g->lcap2 = (uint32_t)cap;
     g->listed = 0;
     g->ftiles = (uint32_t)((bucket_elems + kFTile - 1) / kFTile);
     // a coarse bin holds about k / 40 candidates when the window is as wide as a sample of
@@ -1574,69 +1750,35 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     return true;
 }
 
+// Every call of the single-pass path carries a number of its own; a bucket's window counts
+// as published when its S_READY word shows that number (whatever a workspace held before,
+// it is not this call's number; zero is what a finished call leaves behind).
 std::atomic<uint32_t> g_epoch{0x5EED0001u};
 
-// The three launches of the single-pass path, or the one launch that does the same.
-void launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w, bool warm, hipStream_t st) {
+// The two launches of the single-pass path.  False when the grid would not fit.
+bool launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w, hipStream_t st) {
     // the streaming launch: a sample block per bucket, then per bucket its tiles and 64 bin blocks
     const uint64_t blocks = (uint64_t)g.nbuckets * ((uint64_t)g.ftiles + kGroups + 1) + kGroups;
-    if (tuning().topk_fused && blocks < 0x7FFFFFFFull) {
-        uint32_t epoch = ++g_epoch;
-        if (epoch == 0) epoch = ++g_epoch;  // zero is what a finished call leaves in S_READY
-        // 100 MHz ticks a block may wait before it gives up
-        const uint64_t lim = (uint64_t)tuning().topk_barrier_ms * 100000ull;
-        // blocks that are resident from the start of the launch: they wait for the sample blocks
-        static const int per_cu = [] {
-            int n = 0;
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_topk_stream, kBlock, 0) != hipSuccess || n < 1) n = 5;
-            return n;
-        }();
-        const uint32_t first_wave = g.nbuckets + (uint32_t)device_info().num_cus * (uint32_t)per_cu;
-        k_topk_stream<<<(uint32_t)blocks, kBlock, 0, st>>>(bk, g, w, epoch, first_wave, lim);
-        // the select launch, at most kSelBuckets buckets at a time: all its blocks are resident
-        // together, whatever the order in which the hardware dispatches them
-        for (uint32_t b0 = 0; b0 < g.nbuckets; b0 += kSelBuckets) {
-            const uint32_t nb = g.nbuckets - b0 < (uint32_t)kSelBuckets ? g.nbuckets - b0 : (uint32_t)kSelBuckets;
-            k_topk_select<<<dim3(kGroups, nb), kBlock, 0, st>>>(bk, g, w, b0, lim);
-        }
-        return;
+    if (blocks >= 0x7FFFFFFFull) return false;
+    uint32_t epoch = ++g_epoch;
+    if (epoch == 0) epoch = ++g_epoch;
+    // 100 MHz ticks a block may wait before it gives up
+    const uint64_t lim = (uint64_t)tuning().topk_barrier_ms * 100000ull;
+    // blocks that are resident from the start of the launch: they wait for the sample blocks
+    static const int per_cu = [] {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_topk_stream, kBlock, 0) != hipSuccess || n < 1) n = 5;
+        return n;
+    }();
+    const uint32_t first_wave = g.nbuckets + (uint32_t)device_info().num_cus * (uint32_t)per_cu;
+    k_topk_stream<<<(uint32_t)blocks, kBlock, 0, st>>>(bk, g, w, epoch, first_wave, lim);
+    // the select launch, at most kSelBuckets buckets at a time: all its blocks are resident
+    // together, whatever the order in which the hardware dispatches them
+    for (uint32_t b0 = 0; b0 < g.nbuckets; b0 += kSelBuckets) {
+        const uint32_t nb = g.nbuckets - b0 < (uint32_t)kSelBuckets ? g.nbuckets - b0 : (uint32_t)kSelBuckets;
+        k_topk_select<<<dim3(kGroups, nb), kBlock, 0, st>>>(bk, g, w, b0, lim);
     }
-    // the window comes from the previous call's exact threshold when there was one
-    if (!warm) k_topk_sample<<<g.nbuckets, kSampleThreads, 0, st>>>(bk, g, w);
-    const uint32_t atiles = (uint32_t)((g.bucket_elems + kATile - 1) / kATile);
-    k_topk_pass_a_fast<<<dim3(atiles, g.nbuckets), kAThreads, 0, st>>>(bk, g, w);
-    // 100 MHz ticks a block may wait at a barrier before it gives up
-    const uint64_t limit = (uint64_t)tuning().topk_barrier_ms * 100000ull;
-    k_topk_tail<<<dim3(kNSub, g.nbuckets), kBlock, 0, st>>>(bk, g, w, limit);
-}
-
-// Workspaces whose state words hold a window prediction: address -> shape of the last
-// single-pass call that used it.  A call finds its workspace here with the same shape
-// and skips the sample kernel; anything else (first use, another shape, the exact path
-// in between, mccl_hip_topk_workspace_forget) starts from a fresh sample.
-struct WarmShape {
-    uint64_t n_total, bucket_elems;
-    double ratio;
-    int device;
-};
-std::mutex g_warm_mu;
-std::unordered_map<uintptr_t, WarmShape> g_warm;
-
-bool take_warm(void* workspace, const Geometry& g, double ratio, bool single_pass) {
-    std::lock_guard<std::mutex> lock(g_warm_mu);
-    const uintptr_t key = (uintptr_t)workspace;
-    if (!single_pass) {
-        g_warm.erase(key);
-        return false;
-    }
-    const WarmShape now = {g.n_total, g.bucket_elems, ratio, device_info().device};
-    auto it = g_warm.find(key);
-    const bool warm = it != g_warm.end() && it->second.n_total == now.n_total &&
-                      it->second.bucket_elems == now.bucket_elems && it->second.ratio == now.ratio &&
-                      it->second.device == now.device;
-    if (g_warm.size() > 4096 && it == g_warm.end()) g_warm.clear();
-    g_warm[key] = now;
-    return warm;
+    return true;
 }
 
 }  // namespace
@@ -1645,13 +1787,6 @@ bool take_warm(void* workspace, const Geometry& g, double ratio, bool single_pas
 using namespace mcclhip;
 
 extern "C" {
-
-int mccl_hip_topk_workspace_forget(void* workspace) {
-    if (!workspace) return MCCL_HIP_ERR_ARG;
-    std::lock_guard<std::mutex> lock(g_warm_mu);
-    g_warm.erase((uintptr_t)workspace);
-    return MCCL_HIP_OK;
-}
 
 uint32_t mccl_hip_topk_k(uint64_t count, double ratio) {
     uint32_t k = static_cast<uint32_t>(static_cast<double>(count) * ratio);
@@ -1674,7 +1809,7 @@ uint64_t mccl_hip_topk_workspace_bytes(uint64_t n_total, uint64_t bucket_elems, 
 int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
                            uint64_t bucket_elems, double ratio, void* wire,
                            uint64_t wire_stride, void* workspace, uint64_t workspace_bytes,
-                           void* stream) {
+                           int* status, void* stream) {
     if (!grad || !residual || !wire || !workspace) return MCCL_HIP_ERR_ARG;
     if (!(ratio > 0.0 && ratio <= 1.0)) return MCCL_HIP_ERR_ARG;
     Geometry g;
@@ -1689,8 +1824,9 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     // the carved arrays are 16-byte aligned inside the caller's buffer
     void* aligned = (void*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
     Workspace w = carve(aligned, g);
-    const int path = tuning().topk_path;  // 0 auto, 1 exact path only, 2 fast path at any size
-    const bool fast = path == 2 || (path == 0 && g.bucket_elems >= kFastMinBucket);
+    w.status = status;
+    const int path = tuning().topk_path;  // 0 auto, 1 exact path only, 2 single-pass path at any size
+    bool fast = path == 2 || (path == 0 && g.bucket_elems >= kFastMinBucket);
 
     const uint64_t cap = (uint64_t)device_info().num_cus * (uint64_t)tuning().fold_blocks_per_cu;
     const uint64_t nvec = g.bucket_elems / 4;
@@ -1698,15 +1834,15 @@ int mccl_hip_topk_compress(const float* grad, float* residual, uint64_t n_total,
     const uint64_t need_r = (nvec + kBlock * 4 - 1) / (kBlock * 4);
     const uint32_t bx_r = clamp_u32(bx < need_r ? bx : need_r, 1, 65535);
     const uint32_t bx_t = clamp_u32(bx < g.tiles ? bx : g.tiles, 1, 65535);
-    const bool warm = take_warm(workspace, g, ratio, fast) && tuning().topk_warm != 0;
     if (fast) {
         Buckets bk = {};
         bk.grad = grad;
         bk.residual = residual;
         bk.wire = (uint8_t*)wire;
         bk.wire_stride = wire_stride;
-        launch_single_pass(bk, g, w, warm, st);
-    } else {
+        fast = launch_single_pass(bk, g, w, st);
+    }
+    if (!fast) {
         const uint64_t zw = zeroed_words(g);
         k_zero_words<<<clamp_u32((zw / 4 + kBlock - 1) / kBlock, 1, cap), kBlock, 0, st>>>(w.hist, zw);
         const uint64_t need_a = (nvec + kBlock * 2 - 1) / (kBlock * 2);
@@ -1733,7 +1869,7 @@ uint64_t mccl_hip_topk_list_workspace_bytes(const uint64_t* host_counts, uint32_
 int mccl_hip_topk_compress_list(const float* const* host_grads, float* const* host_residuals,
                                 const uint64_t* host_counts, void* const* host_wires,
                                 const uint64_t* host_wire_capacities, uint32_t nbuckets, double ratio,
-                                void* workspace, uint64_t workspace_bytes, void* stream) {
+                                void* workspace, uint64_t workspace_bytes, int* status, void* stream) {
     if (!host_grads || !host_residuals || !host_counts || !host_wires || !host_wire_capacities || !workspace)
         return MCCL_HIP_ERR_ARG;
     if (nbuckets == 0 || nbuckets > kMaxListed || !(ratio > 0.0 && ratio <= 1.0)) return MCCL_HIP_ERR_ARG;
@@ -1760,9 +1896,8 @@ int mccl_hip_topk_compress_list(const float* const* host_grads, float* const* ho
     if (rc) return rc;
     void* aligned = (void*)(((uintptr_t)workspace + 15) & ~(uintptr_t)15);
     Workspace w = carve(aligned, g);
-    // a list changes from call to call: every call samples
-    mccl_hip_topk_workspace_forget(workspace);
-    launch_single_pass(bk, g, w, false, (hipStream_t)stream);
+    w.status = status;
+    if (!launch_single_pass(bk, g, w, (hipStream_t)stream)) return MCCL_HIP_ERR_ARG;
     return launch_status();
 }
 
@@ -1788,3 +1923,4 @@ int mccl_hip_topk_path_report(const void* workspace, uint64_t n_total, uint64_t 
 }
 
 }  // extern "C"
+

@@ -114,16 +114,15 @@ def topk_workspace(n_total: int, bucket_elems: int, ratio: float, device) -> tor
     nbytes = int(_lib.load().mccl_hip_topk_workspace_bytes(n_total, bucket_elems, ratio))
     if nbytes == 0:
         raise _lib.MCCLHipError(-6, "topk_workspace_bytes")
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-    # the allocator may hand out an address an earlier workspace lived at
-    _lib.load().mccl_hip_topk_workspace_forget(ws.data_ptr())
-    return ws
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
 def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
                   bucket_elems: Optional[int] = None, wire: Optional[torch.Tensor] = None,
-                  workspace: Optional[torch.Tensor] = None, wire_stride: Optional[int] = None):
-    """Returns (wire uint8 tensor [nbuckets * stride], stride). residual is updated."""
+                  workspace: Optional[torch.Tensor] = None, wire_stride: Optional[int] = None,
+                  status: Optional[torch.Tensor] = None):
+    """Returns (wire uint8 tensor [nbuckets * stride], stride). residual is updated.
+    status: int32 device tensor of one element that receives ERR_TIMEOUT (caller zeroes it)."""
     _dev(grad, "grad"); _dev(residual, "residual")
     if grad.dtype != torch.float32 or residual.dtype != torch.float32:
         raise _lib.MCCLHipError(-2, "TopK compression currently supports float32 only")
@@ -139,15 +138,19 @@ def topk_compress(grad: torch.Tensor, residual: torch.Tensor, ratio: float,
         workspace = topk_workspace(max(n, 1), be, ratio, grad.device)
     _dev(wire, "wire", torch.uint8, nb * stride)
     _dev(workspace, "workspace", torch.uint8)
+    if status is not None:
+        _dev(status, "status", torch.int32, 1)
     rc = _lib.load().mccl_hip_topk_compress(grad.data_ptr(), residual.data_ptr(), n, be, ratio,
                                            wire.data_ptr(), stride, workspace.data_ptr(),
-                                           workspace.numel(), _stream())
+                                           workspace.numel(), status.data_ptr() if status is not None else None,
+                                           _stream())
     _lib.check(rc, "topk_compress")
     return wire, stride
 
 
 def topk_compress_list(grads: Sequence[torch.Tensor], residuals: Sequence[torch.Tensor], ratio: float,
-                       wires: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None):
+                       wires: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None,
+                       status: Optional[torch.Tensor] = None):
     """Top-k payloads of a list of separate buckets in one call; returns the list of wire tensors
     (each max_compressed_size bytes, the payload at its front).  residuals are updated."""
     nb = len(grads)
@@ -170,15 +173,13 @@ def topk_compress_list(grads: Sequence[torch.Tensor], residuals: Sequence[torch.
             raise _lib.MCCLHipError(-6, "topk_list_workspace_bytes")
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=grads[0].device)
     _dev(workspace, "workspace", torch.uint8)
+    if status is not None:
+        _dev(status, "status", torch.int32, 1)
     rc = _lib.load().mccl_hip_topk_compress_list(_ptrs(grads), _ptrs(residuals), counts, _ptrs(wires), caps, nb,
-                                                ratio, workspace.data_ptr(), workspace.numel(), _stream())
+                                                ratio, workspace.data_ptr(), workspace.numel(),
+                                                status.data_ptr() if status is not None else None, _stream())
     _lib.check(rc, "topk_compress_list")
     return list(wires)
-
-
-def topk_workspace_forget(workspace: torch.Tensor) -> None:
-    """The next compress call with this workspace samples the gradient afresh."""
-    _lib.check(_lib.load().mccl_hip_topk_workspace_forget(workspace.data_ptr()), "topk_workspace_forget")
 
 
 def topk_path_report(workspace: torch.Tensor, n_total: int, bucket_elems: int, ratio: float):
