@@ -607,7 +607,8 @@ constexpr int kFWaves = kBlock / kWave;       // 4
 constexpr int kFTile = kFRegion * kFWaves;    // elements per streaming block
 constexpr int kFVecs = kFRegion / (kWave * 4);  // 16-byte vectors per lane and array: all issued at once
 constexpr int kTileSlots = 128;               // candidate slots per tile
-constexpr int kCoarse = 64;                   // coarse window bins; the last one holds keys >= hi
+constexpr int kCoarse = 128;                  // coarse window bins; the last one holds keys >= hi
+constexpr int kBinsPerLane = kCoarse / kWave; // 2
 constexpr int kGroups = 64;                   // at most this many groups of tiles per bucket
 constexpr int kCntStride = 64;                // words between two groups' arrival counters: 256 bytes, so that the
                                               // arrivals of a bucket's tiles spread over memory channels
@@ -644,11 +645,16 @@ __device__ __forceinline__ u4a load16_agent(const uint32_t* p) {
     asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
     return v;
 }
-// Coarse bins are 2^shift keys wide: the smallest shift that fits [lo, hi) into kCoarse - 1 bins.
-__device__ __forceinline__ uint32_t window_shift(uint32_t lo, uint32_t hi) {
-    uint32_t shift = 0;
-    while (((hi - lo) >> shift) >= (uint32_t)(kCoarse - 1)) shift++;
-    return shift;
+// The kCoarse - 1 bins below the top one divide [lo, hi) evenly: bin = ((key - lo) * mul) >> 32.
+__device__ __forceinline__ uint32_t window_mul(uint32_t lo, uint32_t hi) {
+    const uint32_t range = hi - lo;  // key - lo < range for every key below hi
+    if (range <= (uint32_t)(kCoarse - 1)) return 0xFFFFFFFFu;  // a bin per key
+    return (uint32_t)((((uint64_t)(kCoarse - 1)) << 32) / range);
+}
+// The smallest key of bin j (1 <= j <= kCoarse - 1; bin 0 starts at lo): lo + ceil(j * 2^32 / mul).
+__device__ __forceinline__ uint32_t window_bin_lo(uint32_t lo, uint32_t mul, uint32_t j) {
+    if (j == 0) return lo;
+    return lo + (uint32_t)((((uint64_t)j << 32) + mul - 1) / mul);
 }
 
 struct FusedGeo {       // per-bucket tiling, derived the same way by every block
@@ -669,8 +675,8 @@ __device__ __forceinline__ FusedGeo fused_geo(const Geometry& g, BucketsArg bk, 
 }
 
 // Coarse window bin of a candidate key (key >= lo).
-__device__ __forceinline__ uint32_t coarse_bin(uint32_t key, uint32_t lo, uint32_t hi, uint32_t shift) {
-    return key >= hi ? (uint32_t)(kCoarse - 1) : (key - lo) >> shift;
+__device__ __forceinline__ uint32_t coarse_bin(uint32_t key, uint32_t lo, uint32_t hi, uint32_t mul) {
+    return key >= hi ? (uint32_t)(kCoarse - 1) : __umulhi(key - lo, mul);
 }
 
 // Waits until *p == want.  Called by a whole wavefront or a single thread; false when the wait timed out.
@@ -737,8 +743,7 @@ struct StreamLds {
 };
 struct SelectLds {
     uint32_t lh[kBins0];                 // radix rounds, tie-break, exact fallback
-    // dense_tile_walk's staging area, one per wavefront; the threshold bin's list in between
-    uint32_t dbuf[kFWaves][16 * kWave] __attribute__((aligned(8)));
+    uint32_t dbuf[kFWaves][16 * kWave];  // dense_tile_walk's staging area, one per wavefront
     uint32_t part[kFWaves][kCoarse];
     uint32_t rcnt[kFWaves][kHeld];
     uint32_t wtot[kFWaves];
@@ -802,6 +807,9 @@ __device__ __forceinline__ void sample_pick(const uint32_t* const (&h)[NR], cons
 __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, const Workspace& w, uint32_t b,
                                              uint32_t epoch, StreamLds& L) {
     const FusedGeo fg = fused_geo(g, bk, b);
+#if FUSED_TRACE == 1
+    const uint32_t tr_s0 = (uint32_t)wall_clock64();
+#endif
     const uint64_t bn = fg.bn;
     const float* gp = bucket_grad(g, bk, b);
     const float* rp = bucket_residual(g, bk, b);
@@ -855,6 +863,9 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
     const bool active[NR] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S, rank[2] <= S};
     uint32_t prefix[NR];
     __syncthreads();
+#if FUSED_TRACE == 1
+    const uint32_t tr_s1 = (uint32_t)wall_clock64();
+#endif
     // round 0: key[30:20], one histogram for all ranks
 #pragma unroll
     for (int j = 0; j < PV; j++)
@@ -873,6 +884,9 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         rank[z] = L.s.res[z][1];
     }
     __syncthreads();
+#if FUSED_TRACE == 1
+    const uint32_t tr_s2 = (uint32_t)wall_clock64();
+#endif
     // round 1: key[19:10] among the keys that share a rank's first digit
     {
         const u4a z = {0u, 0u, 0u, 0u};
@@ -906,6 +920,9 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         if (that < lo) that = lo;
         // every store above must have arrived before the window is published
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#if FUSED_TRACE == 1
+        st[25] = tr_s0; st[27] = tr_s1; st[28] = tr_s2; st[26] = (uint32_t)wall_clock64();
+#endif
         store16_agent(st + S_LO_KEY, u4a{lo, hi, that, epoch});
     }
     // off the critical path: the histograms of the exact selection, should the select launch need it
@@ -1046,7 +1063,10 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
             return;
         }
     }
-    const uint32_t lo = L.e.win[0], hi = L.e.win[1], shift = window_shift(L.e.win[0], L.e.win[1]);
+    const uint32_t lo = L.e.win[0], hi = L.e.win[1], wmul = window_mul(L.e.win[0], L.e.win[1]);
+#if FUSED_TRACE == 1
+    if (threadIdx.x == 0) w.blk_eq[(uint64_t)b * kGroups + grp] = (uint32_t)wall_clock64();
+#endif
     const uint64_t bn = fg.bn;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
@@ -1055,16 +1075,17 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
     G.load(g, w, b, grp, fg);
     // candidates per coarse bin
     if (threadIdx.x < kCoarse) L.e.cnt[threadIdx.x] = 0;
+    static_assert(kCoarse <= kBlock, "one thread per coarse bin");
     __syncthreads();
     G.sweep([&](uint32_t, uint32_t, uint32_t cnt, uint64_t a0, uint64_t a1) {
-                if ((uint32_t)lane < cnt) atomicAdd(&L.e.cnt[coarse_bin(key64(a0), lo, hi, shift)], 1u);
-                if ((uint32_t)(kWave + lane) < cnt) atomicAdd(&L.e.cnt[coarse_bin(key64(a1), lo, hi, shift)], 1u);
+                if ((uint32_t)lane < cnt) atomicAdd(&L.e.cnt[coarse_bin(key64(a0), lo, hi, wmul)], 1u);
+                if ((uint32_t)(kWave + lane) < cnt) atomicAdd(&L.e.cnt[coarse_bin(key64(a1), lo, hi, wmul)], 1u);
             },
             [&](uint32_t, uint32_t t) {
                 dense_tile_walk<true>(rp, bn, t, L.e.dbuf[wave], [&](uint32_t, uint32_t v, bool in) {
                     const uint32_t key = v & 0x7FFFFFFFu;
                     const bool cand = in && key >= lo;
-                    wave_hist_add(L.e.cnt, cand, cand ? coarse_bin(key, lo, hi, shift) : 0u);
+                    wave_hist_add(L.e.cnt, cand, cand ? coarse_bin(key, lo, hi, wmul) : 0u);
                 });
             });
     __syncthreads();
@@ -1086,16 +1107,20 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
         }
     };
     G.sweep([&](uint32_t, uint32_t, uint32_t cnt, uint64_t a0, uint64_t a1) {
-                put((uint32_t)lane < cnt, coarse_bin(key64(a0), lo, hi, shift), a0);
-                put((uint32_t)(kWave + lane) < cnt, coarse_bin(key64(a1), lo, hi, shift), a1);
+                put((uint32_t)lane < cnt, coarse_bin(key64(a0), lo, hi, wmul), a0);
+                put((uint32_t)(kWave + lane) < cnt, coarse_bin(key64(a1), lo, hi, wmul), a1);
             },
             [&](uint32_t, uint32_t t) {
                 dense_tile_walk<true>(rp, bn, t, L.e.dbuf[wave], [&](uint32_t i, uint32_t v, bool in) {
                     const uint32_t key = v & 0x7FFFFFFFu;
                     const bool cand = in && key >= lo;
-                    put(cand, cand ? coarse_bin(key, lo, hi, shift) : 0u, (uint64_t)i | ((uint64_t)v << 32));
+                    put(cand, cand ? coarse_bin(key, lo, hi, wmul) : 0u, (uint64_t)i | ((uint64_t)v << 32));
                 });
             });
+#if FUSED_TRACE == 1
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (threadIdx.x == 0) w.grp_cnt[((uint64_t)b * kGroups + grp) * kCntStride + 1] = (uint32_t)wall_clock64();
+#endif
 }
 
 // ---- the streaming launch ------------------------------------------------------------------
@@ -1124,8 +1149,14 @@ __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, 
         b -= 1;
         emit = true;
     }
+#if FUSED_TRACE == 1
+    const uint32_t tr_start = (uint32_t)wall_clock64();
+#endif
     const FusedGeo fg = fused_geo(g, bk, b);
     if (emit) {
+#if FUSED_TRACE == 1
+        if (threadIdx.x == 0 && t < fg.ng) w.blk_above[(uint64_t)b * kGroups + t] = tr_start;
+#endif
         if (t < fg.ng) fused_bin(bk, g, w, b, t, fg, epoch, limit_ticks, L);
         return;
     }
@@ -1163,6 +1194,9 @@ __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, 
     __syncthreads();
     const bool ready = L.a.win[3] != 0;
     const uint32_t lo_key = L.a.win[0], that_key = L.a.win[2];
+#if FUSED_TRACE == 1
+    const uint32_t tr_ready = (uint32_t)wall_clock64();
+#endif
     // both the same in every lane, and kept in scalar registers by saying so at every update
     uint32_t staged = 0;  // candidates of the region so far
     uint32_t dense = 0;   // 1: more candidates than slots
@@ -1287,6 +1321,13 @@ __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, 
     // ---- the block counts itself into its group once all its stores have arrived ----------
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+#if FUSED_TRACE == 1
+    if (threadIdx.x == 0) {
+        w.tile_gt[(uint64_t)b * g.tiles + t] = tr_start;
+        w.tile_eq[(uint64_t)b * g.tiles + t] = (uint32_t)wall_clock64();
+        ((uint32_t*)w.blist)[(uint64_t)b * g.tiles + t] = tr_ready;
+    }
+#endif
     if (threadIdx.x == 0)
         __hip_atomic_fetch_add(w.grp_cnt + ((uint64_t)b * kGroups + t / fg.tpg) * kCntStride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -1463,13 +1504,32 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
     const uint32_t b = first_bucket + blockIdx.y, grp = blockIdx.x;
     const FusedGeo fg = fused_geo(g, bk, b);
     if (grp >= fg.ng) return;
+#if FUSED_TRACE == 2
+    uint32_t* tr = w.tile_gt + (uint64_t)b * g.tiles + grp * 8;
+    if (threadIdx.x == 0) tr[0] = (uint32_t)wall_clock64();
+#define TR(i) do { if (threadIdx.x == 0) tr[i] = (uint32_t)wall_clock64(); } while (0)
+#else
+#define TR(i) do {} while (0)
+#endif
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     uint32_t* out = bucket_wire(g, bk, b);
-    if (st[S_TIMEOUT]) return;  // the streaming launch gave the bucket up: its payload header says so
-    if (grp == 0 && threadIdx.x == 0) st[S_READY] = 0u;  // a replay of a captured launch carries the same epoch
+    // every load of the first round trip is issued before the first value is looked at
     GroupTiles<false> G;
     G.load(g, w, b, grp, fg);
-    const uint32_t lo = st[S_LO_KEY], that_key = st[S_THAT], shift = window_shift(lo, st[S_HI_KEY]);
+    const u4a win = *(const u4a*)(st + S_LO_KEY);
+    const uint32_t gave_up = st[S_TIMEOUT];
+    constexpr int GPW = kGroups / NW;
+    u2a gh[GPW];  // thread (wave, lane): bins 2 lane and 2 lane + 1 of groups [16 wave, 16 wave + 16)
+    static_assert(kBinsPerLane == 2, "a lane owns two neighbouring bins");
+#pragma unroll
+    for (int i = 0; i < GPW; i++) {
+        const uint32_t gi = (uint32_t)((threadIdx.x / kWave) * GPW + i);
+        gh[i] = gi < fg.ng ? *(const u2a*)(w.ghist + ((uint64_t)b * kGroups + gi) * kCoarse + 2 * (threadIdx.x & (kWave - 1)))
+                           : u2a{0u, 0u};
+    }
+    if (gave_up) return;  // the streaming launch gave the bucket up: its payload header says so
+    if (grp == 0 && threadIdx.x == 0) st[S_READY] = 0u;  // a replay of a captured launch carries the same epoch
+    const uint32_t lo = win[0], that_key = win[2], wmul = window_mul(win[0], win[1]);
     const uint32_t k = fg.k;
     const uint64_t bn = fg.bn;
     const int lane = threadIdx.x & (kWave - 1);
@@ -1480,42 +1540,40 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
     bool failed = false;
     do {
     // ---- 3: threshold bin from the groups' counts -------------------------------------------
-    // thread (wave, lane): bin `lane` of groups [16 wave, 16 wave + 16)
-    constexpr int GPW = kGroups / NW;
-    uint32_t gh[GPW];
-    uint32_t mine = 0;
+    u2a mine = {0u, 0u};
 #pragma unroll
-    for (int i = 0; i < GPW; i++) {
-        const uint32_t gi = (uint32_t)(wave * GPW + i);
-        gh[i] = gi < fg.ng ? w.ghist[((uint64_t)b * kGroups + gi) * kCoarse + lane] : 0u;
-        mine += gh[i];
-    }
-    L.part[wave][lane] = mine;
+    for (int i = 0; i < GPW; i++) mine += gh[i];
+    *(u2a*)&L.part[wave][2 * lane] = mine;
     __syncthreads();
-    // scanned from the top bin downwards: lane l looks at bin 63 - l
-    uint32_t totr = 0;
+    TR(1);
+    // scanned from the top bin downwards: lane l looks at bins 127 - 2 l (first) and 126 - 2 l
+    u2a tot = {0u, 0u};  // tot[0]: bin 126 - 2 l, tot[1]: bin 127 - 2 l
 #pragma unroll
-    for (int i = 0; i < NW; i++) totr += L.part[i][kCoarse - 1 - lane];
-    const uint32_t inc = wave_inclusive_scan(totr);
+    for (int i = 0; i < NW; i++) tot += *(const u2a*)&L.part[i][kCoarse - 2 - 2 * lane];
+    const uint32_t inc = wave_inclusive_scan(tot[0] + tot[1]);
     const uint64_t reach = __ballot(inc >= k);
     if (!reach) {  // fewer than k candidates
         failed = true;
         break;
     }
     const int lstar = __ffsll((long long)reach) - 1;
-    const uint32_t jstar = (uint32_t)(kCoarse - 1 - lstar);
+    const uint32_t pair_hi = (uint32_t)__shfl((int)tot[1], lstar, kWave), pair_lo = (uint32_t)__shfl((int)tot[0], lstar, kWave);
+    const uint32_t above_pair = (uint32_t)__shfl((int)inc, lstar, kWave) - pair_hi - pair_lo;  // candidates in the bins above the pair
+    const bool in_hi = above_pair + pair_hi >= k;                                     // the upper bin of the pair reaches k
+    const uint32_t jstar = (uint32_t)(kCoarse - 1 - 2 * lstar) - (in_hi ? 0u : 1u);
     if (jstar == (uint32_t)(kCoarse - 1)) {  // the threshold lies at or above the window's upper end
         failed = true;
         break;
     }
-    const uint32_t n2 = (uint32_t)__shfl((int)totr, lstar, kWave);          // candidates in the threshold bin
-    const uint32_t above_total = (uint32_t)__shfl((int)inc, lstar, kWave) - n2;
-    const uint32_t need = k - above_total;                                   // picks inside the bin, 1..n2
+    const uint32_t n2 = in_hi ? pair_hi : pair_lo;                     // candidates in the threshold bin
+    const uint32_t above_total = above_pair + (in_hi ? 0u : pair_hi);
+    const uint32_t need = k - above_total;                              // picks inside the bin, 1..n2
     // certain picks (bins above the threshold bin) in the groups before this one
     uint32_t ab = 0;
 #pragma unroll
     for (int i = 0; i < GPW; i++)
-        if ((uint32_t)lane > jstar && (uint32_t)(wave * GPW + i) < grp) ab += gh[i];
+        if ((uint32_t)(wave * GPW + i) < grp)
+            ab += ((uint32_t)(2 * lane) > jstar ? gh[i][0] : 0u) + ((uint32_t)(2 * lane + 1) > jstar ? gh[i][1] : 0u);
     uint32_t above_before;
     block_exclusive_scan(ab, L.scratch, &above_before);
     if (n2 > g.lcapb) {  // more keys in the threshold bin than its list holds (heavy ties, clustered values)
@@ -1525,32 +1583,31 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
 
     // ---- 4: exact threshold from the bin's list ---------------------------------------------
     const uint64_t* l2 = w.blist + ((uint64_t)b * (kCoarse - 1) + jstar) * g.lcapb;
-    // the first 2048 entries are parked in LDS (the dense walks' staging area is idle until the emit)
-    constexpr uint32_t kL2Cached = kFWaves * 16 * kWave / 2;
-    uint64_t* const lcache = (uint64_t*)&L.dbuf[0][0];
-    {
-        constexpr int PER = kL2Cached / kBlock;
-        uint64_t ent[PER];
+    // the first 4096 entries stay in registers (a bin of the expected width holds about 3500)
+    constexpr int kL2Regs = 16;
+    uint64_t ent[kL2Regs];
 #pragma unroll
-        for (int j = 0; j < PER; j++) {
-            const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
-            ent[j] = i < n2 ? l2[i] : 0ull;
-        }
-#pragma unroll
-        for (int j = 0; j < PER; j++) lcache[(uint32_t)j * kBlock + threadIdx.x] = ent[j];  // a thread reads back only what it wrote
+    for (int j = 0; j < kL2Regs; j++) {
+        const uint32_t i = (uint32_t)j * kBlock + threadIdx.x;
+        ent[j] = i < n2 ? l2[i] : 0ull;
     }
     auto for_list2 = [&](auto&& body) {
+#pragma unroll
+        for (int j = 0; j < kL2Regs; j++)
+            if ((uint32_t)j * kBlock + threadIdx.x < n2) body((uint32_t)ent[j], key64(ent[j]));
 #pragma unroll 1
-        for (uint32_t i = threadIdx.x; i < n2; i += kBlock) {
-            const uint64_t e = i < kL2Cached ? lcache[i] : l2[i];
+        for (uint32_t i = kL2Regs * kBlock + threadIdx.x; i < n2; i += kBlock) {
+            const uint64_t e = l2[i];
             body((uint32_t)e, key64(e));
         }
     };
+    TR(2);
     uint32_t* lh = L.lh;
-    const uint32_t bin_lo = lo + (jstar << shift);  // smallest key of the threshold bin
+    const uint32_t bin_lo = window_bin_lo(lo, wmul, jstar);  // smallest key of the threshold bin
+    const uint32_t bin_span = window_bin_lo(lo, wmul, jstar + 1) - bin_lo;  // jstar <= kCoarse - 2
     uint32_t vprefix = 0, want = need;              // key - bin_lo: up to 30 bits, selected as 10 + 10 + 10
-    // a bin spans 2^shift keys: rounds whose digits lie wholly above that are skipped
-    const int first_round = shift <= 10 ? 2 : (shift <= 20 ? 1 : 0);
+    // rounds whose digits lie wholly above the bin's span are skipped
+    const int first_round = bin_span <= (1u << 10) ? 2 : (bin_span <= (1u << 20) ? 1 : 0);
 #pragma unroll 1
     for (int r = first_round; r < 3; r++) {
         const int sh = 20 - 10 * r;
@@ -1572,12 +1629,14 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
         want = left;
     }
     if (failed) break;
+    TR(6);
     const uint32_t T = bin_lo + vprefix;
     const uint32_t need2 = want;
     const uint32_t ties = lh[vprefix & (kBinsR - 1)];
     __syncthreads();
     // when only some keys equal to T are taken, they are the need2 lowest indices
     const uint32_t istar = ties != need2 ? resolve_ties64(l2, n2, T, need2, lh, L.scratch) : 0xFFFFFFFFu;
+    TR(7);
     auto is_pick = [&](bool valid, uint32_t key, uint32_t idx) {
         return valid && (key > T || (key == T && idx <= istar));
     };
@@ -1598,6 +1657,7 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
         break;
     }
 
+    TR(3);
     // ---- 5: payload, in index order -----------------------------------------------------------
     // picks per tile first: the register-held tiles' into rcnt, the others' into the total
     uint32_t w_total = 0;
@@ -1617,6 +1677,7 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
           });
     if (lane == 0) L.wtot[wave] = w_total;
     __syncthreads();
+    TR(4);
     uint32_t wave_off = above_before + l2_before;
     for (int i = 0; i < wave; i++) wave_off += L.wtot[i];
     auto emit_half = [&](bool valid, uint64_t e, uint32_t pos) {
@@ -1691,6 +1752,7 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
             return;
         }
     }
+    TR(5);
     if (grp == 0 && threadIdx.x == 0 && !ld_agent(st + S_TIMEOUT)) out[0] = k;
 }
 
@@ -1742,9 +1804,10 @@ bool make_geometry(uint64_t n_total, uint64_t bucket_elems, double ratio, Geomet
     g->k_last = mccl_hip_topk_k(n_total - (nb - 1) * bucket_elems, ratio);
     g->listed = 0;
     g->ftiles = (uint32_t)((bucket_elems + kFTile - 1) / kFTile);
-    // a coarse bin holds about k / 40 candidates when the window is as wide as a sample of
-    // 8192 leaves it; k / 8 + 2048 entries leave room for uneven bins
-    uint64_t capb = (uint64_t)g->k_full / 8 + 2048;
+    // a coarse bin holds about k / 80 candidates when the window is as wide as a sample of 8192
+    // leaves it, the bins at the window's lower end three times that; k / 10 + 2048 entries
+    // leave room for more uneven ones
+    uint64_t capb = (uint64_t)g->k_full / 10 + 2048;
     if (capb > bucket_elems) capb = bucket_elems;
     g->lcapb = (uint32_t)capb;
     return true;
