@@ -82,8 +82,8 @@ struct Workspace {
     uint32_t* tile_cnt;     // [nbuckets][ftiles] candidates in the tile's slots, or kDense
     uint64_t* slots;        // [nbuckets][ftiles][128] (bits << 32) | index, index order
     uint32_t* grp_cnt;      // [nbuckets][64][kCntStride] finished tiles per group (first word of each 256 bytes)
-    uint32_t* ghist;        // [nbuckets][64 groups][64 bins] candidates per group and coarse window bin
-    uint32_t* bin_fill;     // [nbuckets][64] entries in each coarse bin's list
+    uint32_t* gsuf;         // [nbuckets][128 bins][64 groups] a group's candidates in the bins above bin j
+    uint32_t* bin_fill;     // [nbuckets][128] the bucket's candidates per coarse window bin (= entries of the bin's list)
     uint64_t* blist;        // [nbuckets][63][lcapb] the window's candidates by coarse bin, any order
     int* status;            // caller's device word (may be null): receives MCCL_HIP_ERR_TIMEOUT when a block gives up
 };
@@ -742,9 +742,10 @@ struct StreamLds {
     };
 };
 struct SelectLds {
-    uint32_t lh[kBins0];                 // radix rounds, tie-break, exact fallback
+    uint32_t lh[kBins0] __attribute__((aligned(16)));  // radix rounds, tie-break, exact fallback
     uint32_t dbuf[kFWaves][16 * kWave];  // dense_tile_walk's staging area, one per wavefront
-    uint32_t part[kFWaves][kCoarse];
+    uint32_t wsum[1][kBlock / kWave];
+    uint32_t res[1][2];
     uint32_t rcnt[kFWaves][kHeld];
     uint32_t wtot[kFWaves];
     uint32_t scratch[kBlock / kWave + 2];
@@ -1090,12 +1091,21 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
             });
     __syncthreads();
     if (threadIdx.x < kCoarse) {
+        // the bucket's count per bin; what it held before is where this group's entries go in the
+        // bin's list (the top bin, keys >= hi, holds picks for certain as long as the window holds
+        // and has no list)
         const uint32_t c = L.e.cnt[threadIdx.x];
-        w.ghist[((uint64_t)b * kGroups + grp) * kCoarse + threadIdx.x] = c;
-        // the top bin (keys >= hi) holds picks for certain as long as the window holds: no list
-        L.e.base[threadIdx.x] = (c && threadIdx.x < kCoarse - 1)
-            ? __hip_atomic_fetch_add(w.bin_fill + (uint64_t)b * kCoarse + threadIdx.x, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-            : 0u;
+        L.e.base[threadIdx.x] = c ? __hip_atomic_fetch_add(w.bin_fill + (uint64_t)b * kCoarse + threadIdx.x, c,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                  : 0u;
+    }
+    if (wave == 0) {
+        // this group's candidates above each bin: lane l takes bins 127 - 2 l and 126 - 2 l
+        const uint32_t c_hi = L.e.cnt[kCoarse - 1 - 2 * lane], c_lo = L.e.cnt[kCoarse - 2 - 2 * lane];
+        const uint32_t inc = wave_inclusive_scan(c_hi + c_lo);
+        uint32_t* col = w.gsuf + (uint64_t)b * kCoarse * kGroups + grp;
+        col[(uint64_t)(kCoarse - 1 - 2 * lane) * kGroups] = inc - c_hi - c_lo;
+        col[(uint64_t)(kCoarse - 2 - 2 * lane) * kGroups] = inc - c_lo;
     }
     __syncthreads();
     // binned copies (read by the next launch: plain stores)
@@ -1500,7 +1510,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
                                                            uint64_t limit_ticks) {
     const BucketsArg bk = buckets_arg();
     __shared__ SelectLds L;
-    constexpr int NW = kBlock / kWave;
     const uint32_t b = first_bucket + blockIdx.y, grp = blockIdx.x;
     const FusedGeo fg = fused_geo(g, bk, b);
     if (grp >= fg.ng) return;
@@ -1513,20 +1522,16 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
 #endif
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     uint32_t* out = bucket_wire(g, bk, b);
-    // every load of the first round trip is issued before the first value is looked at
-    GroupTiles<false> G;
-    G.load(g, w, b, grp, fg);
+    // Every load of the first round trip is issued before the first value is looked at, the small
+    // ones first: loads complete in order, and the threshold bin is found (and its list requested)
+    // while the group's slots are still arriving.
     const u4a win = *(const u4a*)(st + S_LO_KEY);
     const uint32_t gave_up = st[S_TIMEOUT];
-    constexpr int GPW = kGroups / NW;
-    u2a gh[GPW];  // thread (wave, lane): bins 2 lane and 2 lane + 1 of groups [16 wave, 16 wave + 16)
     static_assert(kBinsPerLane == 2, "a lane owns two neighbouring bins");
-#pragma unroll
-    for (int i = 0; i < GPW; i++) {
-        const uint32_t gi = (uint32_t)((threadIdx.x / kWave) * GPW + i);
-        gh[i] = gi < fg.ng ? *(const u2a*)(w.ghist + ((uint64_t)b * kGroups + gi) * kCoarse + 2 * (threadIdx.x & (kWave - 1)))
-                           : u2a{0u, 0u};
-    }
+    // scanned from the top bin downwards: lane l looks at bins 127 - 2 l (tot[1]) and 126 - 2 l (tot[0])
+    const u2a tot = *(const u2a*)(w.bin_fill + (uint64_t)b * kCoarse + kCoarse - 2 - 2 * (threadIdx.x & (kWave - 1)));
+    GroupTiles<false> G;
+    G.load(g, w, b, grp, fg);
     if (gave_up) return;  // the streaming launch gave the bucket up: its payload header says so
     if (grp == 0 && threadIdx.x == 0) st[S_READY] = 0u;  // a replay of a captured launch carries the same epoch
     const uint32_t lo = win[0], that_key = win[2], wmul = window_mul(win[0], win[1]);
@@ -1539,17 +1544,8 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
 
     bool failed = false;
     do {
-    // ---- 3: threshold bin from the groups' counts -------------------------------------------
-    u2a mine = {0u, 0u};
-#pragma unroll
-    for (int i = 0; i < GPW; i++) mine += gh[i];
-    *(u2a*)&L.part[wave][2 * lane] = mine;
-    __syncthreads();
+    // ---- 3: threshold bin from the bucket's counts ------------------------------------------
     TR(1);
-    // scanned from the top bin downwards: lane l looks at bins 127 - 2 l (first) and 126 - 2 l
-    u2a tot = {0u, 0u};  // tot[0]: bin 126 - 2 l, tot[1]: bin 127 - 2 l
-#pragma unroll
-    for (int i = 0; i < NW; i++) tot += *(const u2a*)&L.part[i][kCoarse - 2 - 2 * lane];
     const uint32_t inc = wave_inclusive_scan(tot[0] + tot[1]);
     const uint64_t reach = __ballot(inc >= k);
     if (!reach) {  // fewer than k candidates
@@ -1568,14 +1564,9 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
     const uint32_t n2 = in_hi ? pair_hi : pair_lo;                     // candidates in the threshold bin
     const uint32_t above_total = above_pair + (in_hi ? 0u : pair_hi);
     const uint32_t need = k - above_total;                              // picks inside the bin, 1..n2
-    // certain picks (bins above the threshold bin) in the groups before this one
-    uint32_t ab = 0;
-#pragma unroll
-    for (int i = 0; i < GPW; i++)
-        if ((uint32_t)(wave * GPW + i) < grp)
-            ab += ((uint32_t)(2 * lane) > jstar ? gh[i][0] : 0u) + ((uint32_t)(2 * lane + 1) > jstar ? gh[i][1] : 0u);
-    uint32_t above_before;
-    block_exclusive_scan(ab, L.scratch, &above_before);
+    // certain picks (bins above the threshold bin) in the groups before this one: requested now,
+    // summed when the bin's list has been requested as well
+    const uint32_t ab = threadIdx.x < grp ? w.gsuf[((uint64_t)b * kCoarse + jstar) * kGroups + threadIdx.x] : 0u;
     if (n2 > g.lcapb) {  // more keys in the threshold bin than its list holds (heavy ties, clustered values)
         failed = true;
         break;
@@ -1601,6 +1592,8 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
             body((uint32_t)e, key64(e));
         }
     };
+    uint32_t above_before;
+    block_exclusive_scan(ab, L.scratch, &above_before);
     TR(2);
     uint32_t* lh = L.lh;
     const uint32_t bin_lo = window_bin_lo(lo, wmul, jstar);  // smallest key of the threshold bin
@@ -1619,8 +1612,13 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
             if ((v >> hs) == (vprefix >> hs)) atomicAdd(&lh[(v >> sh) & (kBinsR - 1)], 1u);
         });
         __syncthreads();
-        uint32_t left;
-        const uint32_t bin = pick_bin<kBinsR, kBlock>(lh, want, 0, &left, L.scratch);
+        {
+            const uint32_t* const hists[1] = {lh};
+            const uint32_t wants[1] = {want};
+            sample_pick<kBinsR, 1>(hists, wants, L.wsum, L.res);
+        }
+        const uint32_t bin = L.res[0][0], left = L.res[0][1];
+        __syncthreads();  // res is rewritten by the next round
         if (bin >= (uint32_t)kBinsR) {  // the list holds fewer matching keys than the counts promised
             failed = true;
             break;
@@ -1767,7 +1765,7 @@ uint64_t zeroed_words(const Geometry& g) {
 uint64_t workspace_words(const Geometry& g) {
     return zeroed_words(g) + 2 * align4((uint64_t)g.nbuckets * g.tiles) + 2 * align4((uint64_t)g.nbuckets * kGroups) +
            align4((uint64_t)g.nbuckets * g.ftiles) + align4((uint64_t)g.nbuckets * g.ftiles * kTileSlots * 2) +
-           align4((uint64_t)g.nbuckets * kGroups * kCntStride) + align4((uint64_t)g.nbuckets * kGroups * kCoarse) +
+           align4((uint64_t)g.nbuckets * kGroups * kCntStride) + align4((uint64_t)g.nbuckets * kCoarse * kGroups) +
            align4((uint64_t)g.nbuckets * kCoarse) + align4((uint64_t)g.nbuckets * (kCoarse - 1) * g.lcapb * 2);
 }
 
@@ -1783,7 +1781,7 @@ Workspace carve(void* base, const Geometry& g) {
     w.tile_cnt = p;    p += align4((uint64_t)g.nbuckets * g.ftiles);
     w.slots = (uint64_t*)p;  p += align4((uint64_t)g.nbuckets * g.ftiles * kTileSlots * 2);
     w.grp_cnt = p;     p += align4((uint64_t)g.nbuckets * kGroups * kCntStride);
-    w.ghist = p;       p += align4((uint64_t)g.nbuckets * kGroups * kCoarse);
+    w.gsuf = p;       p += align4((uint64_t)g.nbuckets * kGroups * kCoarse);
     w.bin_fill = p;    p += align4((uint64_t)g.nbuckets * kCoarse);
     w.blist = (uint64_t*)p;
     w.status = nullptr;
