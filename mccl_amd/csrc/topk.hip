@@ -756,17 +756,19 @@ struct SelectLds {
 // For NR ranks at once: the bin in which a top-down scan of histogram h[z] reaches rank[z],
 // and how many of the rank's elements fall inside that bin.  Thread t owns the PER bins below
 // BINS - PER t (16-byte LDS reads).  res[z] = {bin, left}; bin = BINS when the histogram holds
-// fewer than rank[z] elements or rank[z] == 0.  Called by all threads of the block.
-template <int BINS, int NR>
+// fewer than rank[z] elements or rank[z] == 0.  SHARED: all ranks are read off h[0].  Called
+// by all threads of the block.
+template <int BINS, int NR, bool SHARED = false>
 __device__ __forceinline__ void sample_pick(const uint32_t* const (&h)[NR], const uint32_t (&rank)[NR],
                                             uint32_t (*wsum)[kBlock / kWave], uint32_t (*res)[2]) {
     constexpr int PER = BINS / kBlock;
+    constexpr int NH = SHARED ? 1 : NR;  // histograms actually scanned
     static_assert(PER % 4 == 0, "16-byte LDS reads");
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
-    uint32_t c[NR][PER], sum[NR], inc[NR];  // c[z][j]: bin BINS - 1 - PER t - j
+    uint32_t c[NH][PER], sum[NH], inc[NH];  // c[z][j]: bin BINS - 1 - PER t - j
 #pragma unroll
-    for (int z = 0; z < NR; z++) {
+    for (int z = 0; z < NH; z++) {
         const u4a* row = (const u4a*)&h[z][BINS - PER * (threadIdx.x + 1)];
         sum[z] = 0;
 #pragma unroll
@@ -783,19 +785,26 @@ __device__ __forceinline__ void sample_pick(const uint32_t* const (&h)[NR], cons
     }
     if (threadIdx.x < NR) { res[threadIdx.x][0] = BINS; res[threadIdx.x][1] = 0; }
     __syncthreads();
+    uint32_t above0[NH];
 #pragma unroll
-    for (int z = 0; z < NR; z++) {
-        uint32_t above = inc[z] - sum[z];
+    for (int z = 0; z < NH; z++) {
+        above0[z] = inc[z] - sum[z];
 #pragma unroll
         for (int i = 0; i < kBlock / kWave; i++)
-            if (i < wave) above += wsum[z][i];
+            if (i < wave) above0[z] += wsum[z][i];
+    }
+#pragma unroll
+    for (int z = 0; z < NR; z++) {
+        constexpr int zz_shared = 0;
+        const int zh = SHARED ? zz_shared : z;
+        uint32_t above = above0[zh];
 #pragma unroll
         for (int j = 0; j < PER; j++) {
-            if (above < rank[z] && rank[z] <= above + c[z][j]) {
+            if (above < rank[z] && rank[z] <= above + c[zh][j]) {
                 res[z][0] = (uint32_t)(BINS - 1 - PER * (int)threadIdx.x - j);
                 res[z][1] = rank[z] - above;
             }
-            above += c[z][j];
+            above += c[zh][j];
         }
     }
     __syncthreads();
@@ -874,10 +883,13 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         for (int q = 0; q < 4; q++)
             if (key[j][q] != 0xFFFFFFFFu) atomicAdd(&h0[key[j][q] >> 20], 1u);
     __syncthreads();
+#if FUSED_TRACE == 1
+    const uint32_t tr_s3 = (uint32_t)wall_clock64();
+#endif
     {
         const uint32_t* const hs[NR] = {h0, h0, h0};
         const uint32_t want[NR] = {active[0] ? rank[0] : 0u, active[1] ? rank[1] : 0u, active[2] ? rank[2] : 0u};
-        sample_pick<kBins0, NR>(hs, want, L.s.wsum, L.s.res);
+        sample_pick<kBins0, NR, true>(hs, want, L.s.wsum, L.s.res);
     }
 #pragma unroll
     for (int z = 0; z < NR; z++) {
@@ -894,16 +906,25 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         for (int i = threadIdx.x; i < 3 * kBinsR / 4; i += kBlock) ((u4a*)h0)[i] = z;
     }
     __syncthreads();
+    // (three comparisons per key; the few keys that share a rank's first digit take the branch)
+    const uint32_t d0 = active[0] ? prefix[0] >> 20 : 0xFFFFFFFFu, d1 = active[1] ? prefix[1] >> 20 : 0xFFFFFFFFu,
+                   d2 = active[2] ? prefix[2] >> 20 : 0xFFFFFFFFu;
 #pragma unroll
     for (int j = 0; j < PV; j++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const uint32_t kq = key[j][q];
-#pragma unroll
-            for (int z = 0; z < NR; z++)
-                if (active[z] && (kq >> 20) == (prefix[z] >> 20)) atomicAdd(&L.s.lh[z][(kq >> 10) & (kBinsR - 1)], 1u);
+            const uint32_t kq = key[j][q], d = kq >> 20;
+            if (d == d0 || d == d1 || d == d2) {
+                const uint32_t bin = (kq >> 10) & (kBinsR - 1);
+                if (d == d0) atomicAdd(&L.s.lh[0][bin], 1u);
+                if (d == d1) atomicAdd(&L.s.lh[1][bin], 1u);
+                if (d == d2) atomicAdd(&L.s.lh[2][bin], 1u);
+            }
         }
     __syncthreads();
+#if FUSED_TRACE == 1
+    const uint32_t tr_s4 = (uint32_t)wall_clock64();
+#endif
     {
         const uint32_t* const hs[NR] = {L.s.lh[0], L.s.lh[1], L.s.lh[2]};
         const uint32_t want[NR] = {active[0] ? rank[0] : 0u, active[1] ? rank[1] : 0u, active[2] ? rank[2] : 0u};
@@ -922,7 +943,7 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         // every store above must have arrived before the window is published
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #if FUSED_TRACE == 1
-        st[25] = tr_s0; st[27] = tr_s1; st[28] = tr_s2; st[26] = (uint32_t)wall_clock64();
+        st[25] = tr_s0; st[27] = tr_s1; st[28] = tr_s2; st[29] = tr_s3; st[30] = tr_s4; st[26] = (uint32_t)wall_clock64();
 #endif
         store16_agent(st + S_LO_KEY, u4a{lo, hi, that, epoch});
     }
