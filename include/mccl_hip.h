@@ -283,7 +283,9 @@ int mccl_hip_fence_block_stream(uint64_t ticket, void* stream);
 int mccl_hip_sync(void* stream);
 
 /* ---- tuning knobs (benchmarks and tests; defaults need no call) ---------- */
-/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_barrier_ms",
+/* keys: "fold_blocks_per_cu", "nontemporal", "topk_path", "topk_barrier_ms", "topk_stall_test" (tests: 1 makes every wait
+ * of the single-pass top-k path run into its limit, so that the give-up path can be exercised
+ * without a stuck kernel),
  * "sparse_path" (0 auto, 1 tile kernels only), "sparse_run_steps" (0 auto),
  * "fp16_portable" (1: the casts follow the reference's portable branch, FP16Compression.cpp:38-73,:96-111) */
 int mccl_hip_set_tuning(const char* key, int value);

@@ -22,6 +22,7 @@ struct Tuning {
     int fold_blocks_per_cu = 256;  // grid cap of the streaming kernels, in blocks per CU
     int nontemporal = 1;         // 1: streaming loads/stores carry the `nt` hint (+8..12 % on MI355X)
     int topk_path = 0;           // 0 auto, 1 multi-pass exact path only, 2 single-pass path at any size
+    int topk_stall_test = 0;     // tests only: 1 = the sample blocks publish a wrong epoch, so that every wait of the single-pass path runs into its limit
     int topk_barrier_ms = 2000;  // single-pass path: longest wait of a block for another block of its launch
     int fp16_portable = 0;       // FP16 casts: 1 = the reference's portable branch (half subnormals flushed, NaN bits passed through)
     int sparse_path = 0;         // sparse accumulate with a workspace: 0 auto (runs of tiles up to 8 ranks), 1 tile kernels only

@@ -140,6 +140,8 @@ int mccl_hip_set_tuning(const char* key, int value) {
     } else if (!std::strcmp(key, "topk_path")) {
         if (value < 0 || value > 2) return MCCL_HIP_ERR_ARG;
         t.topk_path = value;
+    } else if (!std::strcmp(key, "topk_stall_test")) {
+        t.topk_stall_test = value ? 1 : 0;
     } else if (!std::strcmp(key, "topk_barrier_ms")) {
         if (value < 0 || value > 60000) return MCCL_HIP_ERR_ARG;
         t.topk_barrier_ms = value;
@@ -163,6 +165,7 @@ int mccl_hip_get_tuning(const char* key) {
     if (!std::strcmp(key, "fold_blocks_per_cu")) return t.fold_blocks_per_cu;
     if (!std::strcmp(key, "nontemporal")) return t.nontemporal;
     if (!std::strcmp(key, "topk_path")) return t.topk_path;
+    if (!std::strcmp(key, "topk_stall_test")) return t.topk_stall_test;
     if (!std::strcmp(key, "topk_barrier_ms")) return t.topk_barrier_ms;
     if (!std::strcmp(key, "fp16_portable")) return t.fp16_portable;
     if (!std::strcmp(key, "sparse_path")) return t.sparse_path;

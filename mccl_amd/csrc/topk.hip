@@ -1156,11 +1156,12 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
 
 // ---- the streaming launch ------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, Workspace w, uint32_t epoch,
-                                                        uint32_t first_wave, uint64_t limit_ticks) {
+                                                        uint32_t published, uint32_t first_wave,
+                                                        uint64_t limit_ticks) {
     const BucketsArg bk = buckets_arg();
     __shared__ StreamLds L;
     if (blockIdx.x < g.nbuckets) {
-        fused_sample(bk, g, w, blockIdx.x, epoch, L);
+        fused_sample(bk, g, w, blockIdx.x, published, L);
         return;
     }
     // segment s of the grid: the tiles of bucket s, then the bin blocks of bucket s - 1 (whose
@@ -1853,7 +1854,9 @@ bool launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w
         return n;
     }();
     const uint32_t first_wave = g.nbuckets + (uint32_t)device_info().num_cus * (uint32_t)per_cu;
-    k_topk_stream<<<(uint32_t)blocks, kBlock, 0, st>>>(bk, g, w, epoch, first_wave, lim);
+    // (tests of the give-up path: the sample blocks publish a number nobody waits for)
+    const uint32_t published = tuning().topk_stall_test ? ~epoch : epoch;
+    k_topk_stream<<<(uint32_t)blocks, kBlock, 0, st>>>(bk, g, w, epoch, published, first_wave, lim);
     // the select launch, at most kSelBuckets buckets at a time: all its blocks are resident
     // together, whatever the order in which the hardware dispatches them
     for (uint32_t b0 = 0; b0 < g.nbuckets; b0 += kSelBuckets) {

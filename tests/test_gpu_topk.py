@@ -50,7 +50,7 @@ def check_compress(ops, g, r, ratio, be=None, pad=0):
             torch.cuda.synchronize()
             got_res = to_np(dr, F32)
             assert np.array_equal(bits(got_res), bits(want_res)), name
-            assert np.array_equal(to_np(dg, F32), g), name  # gradient untouched
+            assert np.array_equal(bits(to_np(dg, F32)), bits(g)), name  # gradient untouched
             w = wire.cpu().numpy()
             for b, ww in enumerate(want_wires):
                 got = w[b * stride: b * stride + ww.size]
@@ -195,6 +195,154 @@ def test_workspace_with_foreign_contents_is_harmless(ops):
             assert wire.cpu().numpy()[:rc].tobytes() == w.tobytes(), fill
             assert np.array_equal(bits(to_np(dres, F32)), bits(res_o)), fill
             assert ops.topk_path_report(ws, n, n, 0.01) == (1, 1)
+
+
+def _with_bits(x, positions, patterns):
+    v = x.view(np.uint32)
+    v[positions] = np.asarray(patterns, np.uint32)
+    return x
+
+
+def test_compress_orders_nan_and_inf_by_bit_pattern(ops):
+    """Selection orders magnitudes by `bits & 0x7FFFFFFF`: infinities above every finite value,
+    NaN patterns above infinity (by payload), ties to the lower index.  A gradient that carries
+    NaN or inf therefore gives a defined payload, the same on both paths as in the oracle: NaNs
+    spread over the bucket, a NaN inside a cluster of large values (a tile with more candidates
+    than slots), and a threshold that falls among equal NaN patterns (tie-break by index)."""
+    rng = np.random.default_rng(606)
+    n = 400_000
+    qnan, qnan2, neg_qnan, top = 0x7FC00000, 0x7FC00123, 0xFFC00001, 0x7FFFFFFF
+    pinf, ninf = 0x7F800000, 0xFF800000
+    # (a) a few specials spread over the bucket
+    g = student_t(rng, n, ties=0.0)
+    pos = rng.choice(n, 12, replace=False)
+    g = _with_bits(g, pos, [qnan, qnan2, neg_qnan, top, pinf, ninf, qnan, qnan, pinf, neg_qnan, qnan2, ninf])
+    r = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    check_compress(ops, g.copy(), r.copy(), 0.01)
+    # (b) a cluster of large values with NaN and inf in its middle: more candidates than a tile has slots
+    g = student_t(rng, n, ties=0.0) * np.float32(1e-3)
+    g[200_000:203_000] = student_t(rng, 3_000, ties=0.0) * np.float32(50.0)
+    g = _with_bits(g, [200_500, 201_000, 201_001, 202_999], [qnan, pinf, neg_qnan, top])
+    check_compress(ops, g.copy(), np.zeros(n, np.float32), 0.01)
+    # (c) the threshold falls among equal NaN patterns: k = 4000, 6000 identical NaNs, 1000 larger patterns
+    g = student_t(rng, n, ties=0.0)
+    same = rng.choice(n, 6_000, replace=False)
+    g = _with_bits(g, same, np.full(6_000, qnan, np.uint32))
+    bigger = rng.choice(np.setdiff1d(np.arange(n), same), 1_000, replace=False)
+    g = _with_bits(g, bigger, np.full(1_000, qnan2, np.uint32))
+    check_compress(ops, g.copy(), np.zeros(n, np.float32), 0.01)
+    # (d) the same with the threshold among infinities of both signs
+    g = student_t(rng, n, ties=0.0)
+    g = _with_bits(g, same, np.where(rng.random(6_000) < 0.5, pinf, ninf).astype(np.uint32))
+    check_compress(ops, g.copy(), np.zeros(n, np.float32), 0.01)
+
+
+def _state_words(ws, nbuckets):
+    """The per-bucket state words inside a top-k workspace (32 words per bucket, behind the
+    4096-word histograms of all buckets), as a view."""
+    w32 = ws.view(torch.int32)
+    off = (nbuckets * 4096 + 3) & ~3
+    return w32[off: off + nbuckets * 32].view(nbuckets, 32)
+
+
+S_TIMEOUT = 13  # word of a bucket's state that a block sets when it gives up waiting
+
+
+def test_timeout_word_is_reported(ops):
+    """The reporting path without any stuck kernel: the host sets the give-up word of a finished
+    call's workspace, and the path report returns the timeout."""
+    from mccl_amd._lib import MCCLHipError
+    n, be = 1_000_000, 262_144
+    rng = np.random.default_rng(41)
+    ws = ops.topk_workspace(n, be, 0.01, DEV)
+    ops.topk_compress(to_dev(student_t(rng, n), F32), torch.zeros(n, device=DEV), 0.01, bucket_elems=be, workspace=ws)
+    assert ops.topk_path_report(ws, n, be, 0.01) == (4, 4)
+    _state_words(ws, 4)[2, S_TIMEOUT] = 1
+    with pytest.raises(MCCLHipError, match="timed out"):
+        ops.topk_path_report(ws, n, be, 0.01)
+
+
+def test_give_up_path_poisons_the_payload_and_sets_the_status(ops):
+    """Every wait of the single-pass path runs into its limit (the sample blocks are told to
+    publish a number nobody waits for; every kernel still exits normally): the status word
+    receives the timeout, the path report raises, every payload header holds 0xFFFFFFFF, and
+    decompress / sparse accumulate reject such a payload.  The next ordinary call on the same
+    workspace is exact again."""
+    from mccl_amd._lib import MCCLHipError
+    n, be = 1_000_000, 262_144
+    nb = 4
+    rng = np.random.default_rng(42)
+    g = student_t(rng, n)
+    ws = ops.topk_workspace(n, be, 0.01, DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    try:
+        ops.set_tuning("topk_stall_test", 1)
+        ops.set_tuning("topk_barrier_ms", 1)
+        wire, stride = ops.topk_compress(to_dev(g, F32), torch.zeros(n, device=DEV), 0.01, bucket_elems=be,
+                                         workspace=ws, status=status)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_tuning("topk_stall_test", 0)
+        ops.set_tuning("topk_barrier_ms", 2000)
+    assert int(status) == -9   # MCCL_HIP_ERR_TIMEOUT
+    with pytest.raises(MCCLHipError, match="timed out"):
+        ops.topk_path_report(ws, n, be, 0.01)
+    hdr = wire.view(torch.int32)[:: stride // 4][:nb].cpu().numpy().view(np.uint32)
+    assert (hdr == 0xFFFFFFFF).all()
+    dstat = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ops.topk_decompress(wire[:stride], stride, be, status=dstat)
+    assert int(dstat) == oracle.ERR_SIZE
+    dstat.zero_()
+    ops.sparse_accumulate(torch.empty(n, device=DEV), [wire], stride, bucket_elems=be, status=dstat)
+    assert int(dstat) == oracle.ERR_SIZE
+    # the same workspace, an ordinary call
+    status.zero_()
+    res_o = np.zeros(n, np.float32)
+    dres = to_dev(res_o, F32)
+    wire, stride = ops.topk_compress(to_dev(g, F32), dres, 0.01, bucket_elems=be, workspace=ws, status=status)
+    want, want_res = oracle_buckets(g, res_o, 0.01, be)
+    w = wire.cpu().numpy()
+    for b, ww in enumerate(want):
+        assert w[b * stride: b * stride + ww.size].tobytes() == ww.tobytes(), b
+    assert np.array_equal(bits(to_np(dres, F32)), bits(want_res))
+    assert int(status) == 0 and ops.topk_path_report(ws, n, be, 0.01) == (nb, nb)
+
+
+def test_more_buckets_than_the_gpu_holds_blocks_for(ops):
+    """48 buckets of 300,000 elements in one call, and a list of 64 buckets: far more bin and
+    select blocks than are resident at once.  Nothing in the streaming launch waits for a later
+    block, and the select launch goes out in groups of 16 buckets: exact bytes, no give-up."""
+    rng = np.random.default_rng(48)
+    be, nb = 300_000, 48
+    n = be * nb - 12_345
+    g = student_t(rng, n, ties=0.01)
+    res_o = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    want, want_res = oracle_buckets(g, res_o, 0.01, be)
+    dres = to_dev(res_o, F32)
+    ws = ops.topk_workspace(n, be, 0.01, DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    try:
+        ops.set_tuning("topk_path", 2)
+        wire, stride = ops.topk_compress(to_dev(g, F32), dres, 0.01, bucket_elems=be, workspace=ws, status=status)
+        assert ops.topk_path_report(ws, n, be, 0.01) == (nb, nb)
+    finally:
+        ops.set_tuning("topk_path", 0)
+    w = wire.cpu().numpy()
+    for b, ww in enumerate(want):
+        assert w[b * stride: b * stride + ww.size].tobytes() == ww.tobytes(), b
+    assert np.array_equal(bits(to_np(dres, F32)), bits(want_res)) and int(status) == 0
+    # a list of 64 buckets of different lengths
+    sizes = [int(s) for s in rng.integers(200_000, 400_000, 64)]
+    grads = [student_t(rng, m) * np.float32(10.0 ** (i % 3 - 1)) for i, m in enumerate(sizes)]
+    res = [np.zeros(m, np.float32) for m in sizes]
+    dres = [to_dev(r, F32) for r in res]
+    wires = ops.topk_compress_list([to_dev(x, F32) for x in grads], dres, 0.01, status=status)
+    torch.cuda.synchronize()
+    assert int(status) == 0
+    for i, (x, wv) in enumerate(zip(grads, wires)):
+        ww, rc = oracle.topk_compress(x, res[i], 0.01)
+        assert wv.cpu().numpy()[:rc].tobytes() == ww.tobytes(), i
+        assert np.array_equal(bits(to_np(dres[i], F32)), bits(res[i])), i
 
 
 def test_one_large_bucket(ops):
