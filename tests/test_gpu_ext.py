@@ -199,6 +199,32 @@ def test_compressor_errors_and_decompress(k):
         comp.decompress(wire, idx_max)
 
 
+def test_compressor_reports_a_give_up_of_the_compress_launch(k):
+    """compress() is asynchronous; a launch that gives up (every wait forced into its limit from
+    the host, all kernels exit normally) is reported by the calls that wait for the stream:
+    check_compress_status() and decompress() raise, and the payload is rejected."""
+    from mccl_amd import hip_ops as ops
+    C = k["C"]
+    comp = C.TopKCompressor(0.01)
+    g = torch.from_numpy(student_t(np.random.default_rng(3), 400_000)).to(DEV)
+    good = comp.compress(g, stable_id=1)
+    comp.check_compress_status()
+    try:
+        ops.set_tuning("topk_stall_test", 1)
+        ops.set_tuning("topk_barrier_ms", 1)
+        bad = comp.compress(g, stable_id=1)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_tuning("topk_stall_test", 0)
+        ops.set_tuning("topk_barrier_ms", 2000)
+    with pytest.raises(RuntimeError, match="Timeout"):
+        comp.check_compress_status()
+    comp.check_compress_status()   # reported once
+    with pytest.raises(RuntimeError, match="size mismatch"):
+        comp.decompress(bad, 400_000)
+    comp.decompress(good, 400_000)
+
+
 def test_two_bucket_residual_isolation(k):
     # tests/test_compression_e2e.py:33-75: alternate two buckets of very different scale
     # through one compressor; each bucket's residual must only ever see its own gradients.
