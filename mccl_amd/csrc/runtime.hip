@@ -15,7 +15,8 @@
 namespace mcclhip {
 
 namespace {
-std::mutex g_mu;
+std::mutex g_mu;        // device properties, tuning
+std::mutex g_fence_mu;  // the fence ring: never held across a wait for the device
 DeviceInfo g_info;
 Tuning g_tuning;
 thread_local int t_last_hip_error = 0;
@@ -116,12 +117,28 @@ int mccl_hip_pointer_check(const void* ptr, uint64_t nbytes, void** device_ptr) 
             break;
         }
         case hipMemoryTypeManaged:
-            dp = const_cast<void*>(ptr);
-            break;
-        case hipMemoryTypeHost:  // pinned: kernels reach it through its device-side alias
-            dp = attr.devicePointer;
+        case hipMemoryTypeHost: {  // pinned: kernels reach it through its device-side alias
+            dp = attr.type == hipMemoryTypeHost ? attr.devicePointer : const_cast<void*>(ptr);
             if (!dp) return MCCL_HIP_ERR_POINTER;
+            // the whole range must lie inside the allocation, as for device memory; an extent
+            // that cannot be determined is not vouched for
+            hipDeviceptr_t base = nullptr;
+            size_t size = 0;
+            uintptr_t p = (uintptr_t)ptr;
+            e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr);
+            if (e != hipSuccess && dp != ptr) {
+                (void)hipGetLastError();
+                p = (uintptr_t)dp;
+                e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)dp);
+            }
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return MCCL_HIP_ERR_POINTER;
+            }
+            const uintptr_t lo = (uintptr_t)base;
+            if (p < lo || nbytes > size || p - lo > size - nbytes) return MCCL_HIP_ERR_POINTER;
             break;
+        }
         default:
             return MCCL_HIP_ERR_POINTER;
     }
@@ -177,43 +194,59 @@ int mccl_hip_get_tuning(const char* key) {
 
 int mccl_hip_fence_signal(void* stream, uint64_t* ticket) {
     if (!ticket) return MCCL_HIP_ERR_ARG;
-    std::lock_guard<std::mutex> lock(g_mu);
     int dev = -1;
     MCCLHIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxFenceDevices) return MCCL_HIP_ERR_ARG;
-    if (!g_ring[dev]) {
-        hipEvent_t* ring = new hipEvent_t[kRing];
-        for (uint64_t i = 0; i < kRing; i++) {
-            hipError_t e = hipEventCreateWithFlags(&ring[i], hipEventDisableTiming);
-            if (e != hipSuccess) {
+    for (;;) {
+        hipEvent_t old = nullptr;
+        {
+            std::lock_guard<std::mutex> lock(g_fence_mu);
+            if (!g_ring[dev]) {
+                hipEvent_t* ring = new hipEvent_t[kRing];
+                for (uint64_t i = 0; i < kRing; i++) {
+                    hipError_t e = hipEventCreateWithFlags(&ring[i], hipEventDisableTiming);
+                    if (e != hipSuccess) {
+                        record_hip_error(e);
+                        for (uint64_t j = 0; j < i; j++) (void)hipEventDestroy(ring[j]);
+                        delete[] ring;
+                        return MCCL_HIP_ERR_RUNTIME;
+                    }
+                }
+                g_ring[dev] = ring;
+            }
+            const uint64_t t = g_next_ticket.load();
+            const uint64_t slot = t % kRing;
+            // The slot's previous owner (kRing tickets older) leaves the ring here.  "Left the
+            // ring" has to mean "complete" for every later wait on it; with per-step fences that
+            // are waited on promptly it already is.
+            hipError_t e = hipSuccess;
+            if (g_slot_ticket[slot] != 0) {
+                old = g_ring[g_slot_device[slot]][slot];
+                e = hipEventQuery(old);
+            }
+            if (e == hipSuccess) {
+                MCCLHIP_TRY(hipEventRecord(g_ring[dev][slot], (hipStream_t)stream));
+                g_slot_ticket[slot] = t;
+                g_slot_device[slot] = dev;
+                g_next_ticket.store(t + 1);
+                *ticket = t;
+                return MCCL_HIP_OK;
+            }
+            if (e != hipErrorNotReady) {
                 record_hip_error(e);
-                for (uint64_t j = 0; j < i; j++) (void)hipEventDestroy(ring[j]);
-                delete[] ring;
                 return MCCL_HIP_ERR_RUNTIME;
             }
         }
-        g_ring[dev] = ring;
-    }
-    const uint64_t t = g_next_ticket.load();
-    const uint64_t slot = t % kRing;
-    // The slot's previous owner (kRing tickets older) leaves the ring here.  "Left
-    // the ring" has to mean "complete" for every later wait on it, so its event is
-    // drained first; with per-step fences that are waited on promptly it already is.
-    if (g_slot_ticket[slot] != 0) {
-        hipEvent_t old = g_ring[g_slot_device[slot]][slot];
-        hipError_t e = hipEventQuery(old);
-        if (e == hipErrorNotReady) e = hipEventSynchronize(old);
+        // The old owner is still running: wait for it WITHOUT the lock (other threads' signals,
+        // queries and stream waits go on meanwhile; the old owner's stream may itself be waiting
+        // for work another thread has yet to enqueue through this library), then look again:
+        // the ticket counter may have moved on to another slot.
+        hipError_t e = hipEventSynchronize(old);
         if (e != hipSuccess) {
             record_hip_error(e);
             return MCCL_HIP_ERR_RUNTIME;
         }
     }
-    MCCLHIP_TRY(hipEventRecord(g_ring[dev][slot], (hipStream_t)stream));
-    g_slot_ticket[slot] = t;
-    g_slot_device[slot] = dev;
-    g_next_ticket.store(t + 1);
-    *ticket = t;
-    return MCCL_HIP_OK;
 }
 
 // 1 complete, 0 pending (then *ev is the ticket's event), negative on error.  A
@@ -230,7 +263,7 @@ static int fence_state_locked(uint64_t ticket, hipEvent_t* ev) {
 // caller polls, the event then reports the newer ticket, recorded only after
 // this one had completed, so the caller still never returns early.
 static int fence_state(uint64_t ticket, hipEvent_t* ev) {
-    std::lock_guard<std::mutex> lock(g_mu);
+    std::lock_guard<std::mutex> lock(g_fence_mu);
     return fence_state_locked(ticket, ev);
 }
 
@@ -268,7 +301,7 @@ int mccl_hip_fence_wait(uint64_t ticket, int timeout_ms) {
 int mccl_hip_fence_block_stream(uint64_t ticket, void* stream) {
     // under the lock: the wait must be enqueued on this ticket's record, not on a
     // later record of the same event
-    std::lock_guard<std::mutex> lock(g_mu);
+    std::lock_guard<std::mutex> lock(g_fence_mu);
     hipEvent_t ev;
     int st = fence_state_locked(ticket, &ev);
     if (st < 0) return st;

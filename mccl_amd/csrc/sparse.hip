@@ -508,6 +508,10 @@ __global__ __launch_bounds__(kRunWaves * kWave, 4) void k_sparse_accumulate_runs
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         uint32_t prev = lane_value(before[r], 0);
+        // The pair in front of the first window must lie before this run: a position-table entry
+        // that points past the run's first pair (a table left by another call racing on shared
+        // scratch, or sampled from a payload that is not ascending) would drop pairs silently.
+        if (wnext[r] > 0 && kk[r] > 0 && prev >= (uint32_t)e0) bad |= 1ull;
 #pragma unroll
         for (int i = 0; i < kRunWins; i++) {
             const uint32_t base = wnext[r] + (uint32_t)i * kWin;

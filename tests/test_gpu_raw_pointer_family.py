@@ -98,6 +98,11 @@ def test_pageable_host_memory_and_bad_ranges_raise_before_any_launch(C):
     d = torch.ones(1000, device=DEV); s = torch.ones(1 << 20, device=DEV)
     with pytest.raises(RuntimeError, match="not memory a GPU kernel can reach"):
         C._cpu_reduce_op_ptr(d.data_ptr(), s.data_ptr(), 1 << 28, OP_SUM)
+    # ... and past the end of a pinned host allocation (its extent is checked like device memory's)
+    hp = torch.ones(1000).pin_memory()
+    with pytest.raises(RuntimeError, match="not memory a GPU kernel can reach"):
+        C._cpu_reduce_op_ptr(hp.data_ptr(), hp.data_ptr(), 1 << 28, OP_SUM)
+    assert float(hp.sum()) == 1000.0
     with pytest.raises(RuntimeError, match="Unsupported ReduceOp"):
         C._cpu_reduce_op(d, d.clone(), 5)
     with pytest.raises(RuntimeError, match="Shape mismatch"):
