@@ -1,8 +1,10 @@
 """mccl_hip_sparse_accumulate_static (the entry point that allocates nothing: its
 position table is a static device array) against mccl_hip_sparse_accumulate
-with a caller workspace, bit for bit, through the C ABI: two calls in a row,
-the second on a smaller input, so stale contents of the shared array from the
-first call are in place when the second runs."""
+with a caller workspace AND against the oracle, bit for bit, through the C ABI:
+two calls in a row, the second on a smaller input, so stale contents of the
+shared array from the first call are in place when the second runs.  Free device
+memory as the driver reports it must not change across the call (an allocation
+inside the library would not show in torch's own counters)."""
 import ctypes as C
 
 import numpy as np
@@ -21,6 +23,7 @@ def payloads(rng, ws, n, be, ratio):
     stride = 4 + 8 * (int(be * ratio) + 1)
     shared = rng.random(n) < 0.004
     out = []
+    per_bucket = [[] for _ in range(nb)]
     for _ in range(ws):
         g = student_t(rng, n, ties=0.0)
         g[shared] *= 50.0
@@ -29,8 +32,9 @@ def payloads(rng, ws, n, be, ratio):
             s, e = b * be, min(n, (b + 1) * be)
             w, rc = oracle.topk_compress(g[s:e].copy(), np.zeros(e - s, np.float32), ratio)
             buf[b * stride: b * stride + rc] = w
+            per_bucket[b].append(w)
         out.append(torch.from_numpy(buf).to(DEV))
-    return out, stride
+    return out, stride, per_bucket
 
 
 def test_static_scratch_entry_point_matches_workspace_entry_point():
@@ -41,18 +45,26 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
     status = torch.zeros(1, dtype=torch.int32, device=DEV)
     # first a large call (many tiles, 8 ranks), then a smaller one with other bucket geometry
     for ws, n, be, ratio in ((8, 3_000_017, 655_360, 0.01), (3, 200_003, 65_536, 0.02)):
-        wires, stride = payloads(rng, ws, n, be, ratio)
+        wires, stride, per_bucket = payloads(rng, ws, n, be, ratio)
+        want_o = np.empty(n, np.float32)
+        for b, ww in enumerate(per_bucket):
+            s0, e0 = b * be, min(n, (b + 1) * be)
+            acc, rc = oracle.sparse_accumulate(ww, e0 - s0, scale_by=1.0 / ws)
+            assert rc == oracle.OK
+            want_o[s0:e0] = acc
         want = torch.full((n,), 3.0, device=DEV)
         ops.sparse_accumulate(want, wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status,
                               workspace="auto")
         got = torch.full((n,), 5.0, device=DEV)
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         ops.sparse_accumulate_static(got, wires, stride, bucket_elems=be, scale_by=1.0 / ws, status=status)
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before
         assert int(status) == 0
         assert np.array_equal(bits(to_np(got, F32)), bits(to_np(want, F32))), (ws, n, be)
+        assert np.array_equal(bits(to_np(got, F32)), bits(want_o)), (ws, n, be)
     # a shape whose bounds table does not fit the static array is refused, nothing is launched
     ws, n, be = 64, 200_000_000, 100_000_000
     need = lib.mccl_hip_sparse_accumulate_workspace_bytes(n, be, ws)
