@@ -51,7 +51,7 @@ def main() -> int:
     import numpy as np
     import torch
     from mccl_amd import hip_ops as ops
-    from mccl_amd import hbm_traffic
+    import bench_traffic as hbm_traffic
 
     # HBM bytes per launch from the committed counter runs; None (with the reason) when they were
     # taken on other versions of the kernel sources or another workload size
@@ -118,8 +118,8 @@ def main() -> int:
     extra["d2d_copy_GBps"] = rate(8 * N, cpy_ms["avg_ms"])
 
     if a.only in ("all", "fold"):
-        # world sizes the kernel has no compile-time instance for (the reference's tests use 3 and 6)
-        for ws_rt in (3, 6):
+        # other world sizes (the reference's tests use 3 and 6); each has an unrolled instance
+        for ws_rt in (3, 5, 6, 7):
             inv = float(np.float32(1.0 / ws_rt))
             r = stats(gpu_time(lambda: ops.ring_fold(out, ranks[:ws_rt], ops.AVG, ops.RING_BASIC,
                                                      bucket_elems=BUCKET, scale_by=inv))[1])
@@ -214,8 +214,8 @@ def main() -> int:
                                           "bytes": topk_bytes, "buckets": nb, "k_per_bucket": ks[0],
                                           "single_pass_buckets": ops.topk_path_report(wsb, N, BUCKET, 0.01)[0]}
         # second half of the headline metric: same fields as `roofline`, for the whole
-        # compress call (three launches: sample, streaming pass, selection)
-        roofline_topk = {"bound": "hbm", "kernel": "mccl_hip_topk_compress (3 launches, dominant k_topk_pass_a_fast)",
+        # compress call (two launches: streaming with sample and binning, selection)
+        roofline_topk = {"bound": "hbm", "kernel": "mccl_hip_topk_compress (2 launches, dominant k_topk_stream)",
                          "achieved": rate(topk_bytes, tk["avg_ms"]), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": rate(topk_bytes, tk["avg_ms"]) / HBM_PEAK_GBPS,
                          "traffic": traffic["topk_compress"] if traffic else None, "traffic_source": traffic_note,
@@ -241,12 +241,12 @@ def main() -> int:
                              steps=max(3, K // 2))[1])
         extra["config4_15_compress_calls"] = {"ms": per["avg_ms"], "GBps": rate(topk_bytes, per["avg_ms"]),
                                               "frac": rate(topk_bytes, per["avg_ms"]) / HBM_PEAK_GBPS,
-                                              "note": "15 x TopKCompressor::compress, 45 launches: bound by the host's launch rate"}
+                                              "note": "15 x TopKCompressor::compress, 30 launches: bound by launch latency"}
         comp = _C.TopKCompressor(0.01)
         many = stats(gpu_time(lambda: comp.compress_many(bufs, stable_ids=ids))[1])
         extra["config4_compress_many"] = {"ms": many["avg_ms"], "GBps": rate(topk_bytes, many["avg_ms"]),
                                           "frac": rate(topk_bytes, many["avg_ms"]) / HBM_PEAK_GBPS,
-                                          "note": "TopKCompressor::compress_many on the same 15 buffers: 3 launches"}
+                                          "note": "TopKCompressor::compress_many on the same 15 buffers: 2 launches"}
         del comp, bufs
 
         # ---- config 5: decompress-accumulate of 8 ranks' payloads -----------------
@@ -271,6 +271,22 @@ def main() -> int:
                                               "bytes": acc_bytes, "status": int(status),
                                               "traffic": traffic["sparse_accumulate"] if traffic else None,
                                               "traffic_source": traffic_note}
+        # the other kernels of the same entry point: no workspace (block-per-tile kernels that
+        # search the payloads themselves), and 12 ranks (more than the runs-of-tiles kernel takes)
+        sn = stats(gpu_time(lambda: ops.sparse_accumulate(acc, wires, stride, bucket_elems=BUCKET, scale_by=0.125,
+                                                          status=status, workspace=None))[1])
+        extra["config5_sparse_accumulate_no_workspace"] = {"ms": sn["avg_ms"], "GBps": rate(acc_bytes, sn["avg_ms"]),
+                                                           "frac": rate(acc_bytes, sn["avg_ms"]) / HBM_PEAK_GBPS}
+        w12 = wires + wires[:4]
+        b12 = 4 * N + 8 * sum(ks) * 12
+        sws12 = ops.sparse_workspace(N, BUCKET, 12, dev)
+        s12 = stats(gpu_time(lambda: ops.sparse_accumulate(acc, w12, stride, bucket_elems=BUCKET, scale_by=1.0 / 12,
+                                                           status=status, workspace=sws12))[1])
+        extra["sparse_accumulate_12_ranks_tile_kernels"] = {"ms": s12["avg_ms"], "GBps": rate(b12, s12["avg_ms"]),
+                                                            "frac": rate(b12, s12["avg_ms"]) / HBM_PEAK_GBPS, "bytes": b12}
+        cfg5_host = None
+        if not a.no_cpu:
+            cfg5_host = [wv[:stride].cpu().numpy() for wv in wires]   # bucket 0 of every rank, for the CPU leg
 
     if a.only == "all":
         # ---- FP16 compressor casts over the whole gradient (6 B / element each way) ----
@@ -337,6 +353,61 @@ def main() -> int:
                 "GBps": (12 * BUCKET + 8 * 65_536 + 4) / s_ref / 1e9, "ms_per_bucket": s_ref * 1e3,
                 "cores": 1, "kind": "reference",
                 "sample": f"one 25 MiB bucket, {reps} repetitions of the reference's compiled TopKCompressor::compress"}
+
+        if a.only in ("all", "sparse") and cfg5_host is not None:
+            # leg (iii): decompress + accumulate in the reference's form - memset and scatter per rank
+            # (csrc/compression/TopKCompression.cpp:122-152), a dense add per rank and x 1/W
+            # (csrc/backend/ProcessGroupMCCL.cpp:2272-2296) - on bucket 0 of the 8 payloads of config 5
+            use_ref = oracle.RefCompressor.available()
+            refc = oracle.RefCompressor(2, 0.01) if use_ref else None
+            accb = np.zeros(BUCKET, np.float32)
+            kb0 = ops.topk_k(BUCKET, 0.01)
+            t0 = time.perf_counter()
+            reps = 0
+            while time.perf_counter() - t0 < 6.0 and reps < 8:
+                accb[:] = 0.0
+                for hw in cfg5_host:
+                    dense = refc.decompress(hw[:4 + 8 * kb0], BUCKET)[0] if use_ref else oracle.topk_decompress(hw, BUCKET)[0]
+                    oracle.fold2(accb, dense, oracle.F32, oracle.OP_SUM, threads=0)
+                oracle.scale(accb, oracle.F32, 0.125, threads=0)
+                reps += 1
+            s3 = (time.perf_counter() - t0) / reps
+            b3 = 4 * BUCKET + 8 * kb0 * W
+            extra["config5_cpu_reference_form"] = {
+                "GBps": b3 / s3 / 1e9, "ms_per_bucket": s3 * 1e3, "cores": min(8, os.cpu_count() or 1),
+                "kind": "reference" if use_ref else "port", "bytes": b3,
+                "sample": f"bucket 0 of the 8 payloads of config 5, {reps} repetitions: per rank the reference's "
+                          "decompress (memset + scatter, one core) and a dense fold with the reference's job split, "
+                          "then x 1/8; same 4 n + 8 k W numerator as the GPU figure"}
+        if a.only in ("all", "fold"):
+            # cross-check of the fold port with torch's CPU kernels on the same host buffers, in the
+            # same ring-step order and with the same numerator: in-place add_ per fold, mul_ per chunk
+            import torch as _t
+            th = [_t.from_numpy(h) for h in host]
+            t0 = time.perf_counter()
+            reps = 0
+            while time.perf_counter() - t0 < 4.0 and reps < 12:
+                for b in range(nbk):
+                    lo, hi = b * BUCKET, min(cn, (b + 1) * BUCKET)
+                    ce = (hi - lo + W - 1) // W
+                    for c in range(W):
+                        s, e = lo + c * ce, min(hi, lo + (c + 1) * ce)
+                        if s >= e:
+                            continue
+                        part = th[c][s:e]
+                        for j in range(1, W):
+                            local = th[(c + j) % W][s:e]
+                            local.add_(part)
+                            part = local
+                        part.mul_(0.125)
+                reps += 1
+            s4 = (time.perf_counter() - t0) / reps
+            extra["cpu_torch_fold_crosscheck"] = {
+                "GBps": (W + 1) * 4 * cn / s4 / 1e9, "threads": _t.get_num_threads(),
+                "working_set_MiB": W * 4 * cn / 2 ** 20,
+                "sample": f"the cpu_baseline sample ({nbk} buckets x {W} ranks) folded with torch's CPU add_ and "
+                          f"mul_ in the same ring-step order, {reps} repetitions, same 36 B/element numerator; "
+                          "a working set that fits the host's last-level cache is served from it"}
 
     if a.only == "all":
         # ---- step-wise ring driver: 8 ranks, chunked ring allreduce (reduce-scatter folds,

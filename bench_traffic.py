@@ -3,7 +3,7 @@ into ``profiles/hbm_traffic.json``: HBM bytes per launch of the fold, the top-k
 compress call and the sparse accumulate call, each counter scaled by what the
 same counter reads for a device-to-device copy of known size in the same run.
 
-    python -m mccl_amd.hbm_traffic <fetch_counter_collection.csv> <write_counter_collection.csv>
+    python bench_traffic.py <fetch_counter_collection.csv> <write_counter_collection.csv>
 
 ``bench.py`` reads the JSON for its ``roofline.traffic`` fields and only trusts it
 while the kernel sources it was measured on are unchanged (their SHA-256 is
@@ -18,8 +18,8 @@ import os
 import sys
 from collections import defaultdict
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-ROOT = os.path.dirname(HERE)
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HERE = os.path.join(ROOT, "mccl_amd")
 OUT = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 SOURCES = ["common.hip.h", "fold.hip", "topk.hip", "sparse.hip"]
 N_GRAD = 96_510_024
@@ -44,7 +44,7 @@ def per_kernel(path: str, counter: str) -> dict:
             name = row["Kernel_Name"]
             if "k_ring_fold" in name and "k_ring_fold<6, 0, true, 8>" not in name:
                 continue                                  # only the fp32 SUM fold of 8 ranks (config 2)
-            for key in ("k_ring_fold", "k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail", "k_sparse_starts",
+            for key in ("k_ring_fold", "k_topk_stream", "k_topk_select", "k_sparse_starts",
                         "k_sparse_bounds", "k_sparse_accumulate", "copyBuffer"):
                 if key in name:
                     vals[key].append((int(row["Grid_Size"]), float(row["Counter_Value"])))
@@ -89,7 +89,7 @@ def main(argv) -> int:
         "kernels": kernels,
         "calls": {
             "ring_fold_f32_w8": total(["k_ring_fold"]),
-            "topk_compress": total(["k_topk_sample", "k_topk_pass_a_fast", "k_topk_tail"]),
+            "topk_compress": total(["k_topk_stream", "k_topk_select"]),
             "sparse_accumulate": total(["k_sparse_starts", "k_sparse_bounds", "k_sparse_accumulate"]),
         },
     }

@@ -3,7 +3,7 @@
 // W-way fold in ring-step order.
 //
 // All of them are HBM-bound streaming kernels: 256-thread blocks, every lane
-// moves 16 bytes per access (global_load/store_dwordx4), kUnroll independent
+// moves 16 bytes per access (global_load/store_dwordx4), a few independent
 // accesses per operand are issued before the first use, and the grid is sized
 // to keep every CU's wave slots full.  The destination is peeled to 16-byte
 // alignment; sources are read with element alignment only, because chunk views
@@ -22,8 +22,13 @@ namespace mcclhip {
 
 namespace {
 
-constexpr int kUnroll = 4;      // binary folds: vectors in flight per thread and operand
-constexpr int kRingUnroll = 4;  // ring fold: vectors in flight per thread and rank buffer
+// Vectors in flight per thread and operand.  Measured on MI355X over 96.5 M elements (fraction
+// of the 8 TB/s peak): the binary folds are fastest with one (fold 0.81 against 0.78 with four,
+// scale 0.86 against 0.77: a 1024-element tile per block keeps the set of tiles in flight one
+// narrow address front); the ring fold with one for three ranks (0.76 against 0.73), eight for
+// six and seven ranks (0.71 against 0.70) and four otherwise.
+constexpr int kUnroll = 1;
+constexpr int ring_unroll(int ws) { return ws == 3 ? 1 : ((ws == 6 || ws == 7) ? 8 : 4); }
 
 template <bool NT>
 __device__ __forceinline__ u4a load_vec_a(const u4a* p) {
@@ -170,7 +175,7 @@ struct RingPtrs {
 // blockIdx.y = bucket * nchunks + chunk.  Each block row folds one chunk of one
 // bucket, so the first rank of the fold is uniform over the block.
 // WSC > 0 fixes the world size at compile time, so the rank loop unrolls and
-// all WSC * kRingUnroll loads of a thread are in flight together; WSC == 0 reads
+// all WSC * ring_unroll(WSC) loads of a thread are in flight together; WSC == 0 reads
 // it at run time.
 template <int DT, int OP, bool NT, int WSC>
 __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, int ws_rt,
@@ -179,7 +184,7 @@ __global__ __launch_bounds__(kBlock) void k_ring_fold(void* out, RingPtrs ptrs, 
                                                       int apply_scale, int stepwise) {
     constexpr int ES = ElemInfo<DT>::size;
     constexpr int EPV = ElemInfo<DT>::per_vec;
-    constexpr int U = kRingUnroll;
+    constexpr int U = ring_unroll(WSC);
     const int ws = WSC > 0 ? WSC : ws_rt;
     const uint32_t bucket = blockIdx.y / nchunks;
     const uint32_t c = blockIdx.y - bucket * nchunks;
@@ -394,7 +399,8 @@ int launch_ring_t(void* out, const RingPtrs& ptrs, int ws, uint64_t n_total, uin
     constexpr int EPV = ElemInfo<DT>::per_vec;
     const uint64_t bn = bucket_elems < n_total ? bucket_elems : n_total;
     const uint64_t ce = (bn + nchunks - 1) / nchunks;
-    const uint64_t tiles = (ce / EPV + (uint64_t)kBlock * kRingUnroll - 1) / ((uint64_t)kBlock * kRingUnroll);
+    const uint64_t tile_vecs = (uint64_t)kBlock * ring_unroll(ws >= 2 && ws <= 8 ? ws : 0);
+    const uint64_t tiles = (ce / EPV + tile_vecs - 1) / tile_vecs;
     const uint64_t rows = (uint64_t)nchunks * nbuckets;
     // One tile per block, x fastest: blocks are dispatched in address order, so
     // the set of tiles in flight is one contiguous front per rank buffer.  A
