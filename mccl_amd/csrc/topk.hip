@@ -817,9 +817,6 @@ __device__ __forceinline__ void sample_pick(const uint32_t* const (&h)[NR], cons
 __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, const Workspace& w, uint32_t b,
                                              uint32_t epoch, StreamLds& L) {
     const FusedGeo fg = fused_geo(g, bk, b);
-#if FUSED_TRACE == 1
-    const uint32_t tr_s0 = (uint32_t)wall_clock64();
-#endif
     const uint64_t bn = fg.bn;
     const float* gp = bucket_grad(g, bk, b);
     const float* rp = bucket_residual(g, bk, b);
@@ -873,9 +870,6 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
     const bool active[NR] = {rank[0] >= 1u && rank[0] <= S, rank[1] <= S, rank[2] <= S};
     uint32_t prefix[NR];
     __syncthreads();
-#if FUSED_TRACE == 1
-    const uint32_t tr_s1 = (uint32_t)wall_clock64();
-#endif
     // round 0: key[30:20], one histogram for all ranks
 #pragma unroll
     for (int j = 0; j < PV; j++)
@@ -883,9 +877,6 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         for (int q = 0; q < 4; q++)
             if (key[j][q] != 0xFFFFFFFFu) atomicAdd(&h0[key[j][q] >> 20], 1u);
     __syncthreads();
-#if FUSED_TRACE == 1
-    const uint32_t tr_s3 = (uint32_t)wall_clock64();
-#endif
     {
         const uint32_t* const hs[NR] = {h0, h0, h0};
         const uint32_t want[NR] = {active[0] ? rank[0] : 0u, active[1] ? rank[1] : 0u, active[2] ? rank[2] : 0u};
@@ -897,9 +888,6 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         rank[z] = L.s.res[z][1];
     }
     __syncthreads();
-#if FUSED_TRACE == 1
-    const uint32_t tr_s2 = (uint32_t)wall_clock64();
-#endif
     // round 1: key[19:10] among the keys that share a rank's first digit
     {
         const u4a z = {0u, 0u, 0u, 0u};
@@ -922,9 +910,6 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
             }
         }
     __syncthreads();
-#if FUSED_TRACE == 1
-    const uint32_t tr_s4 = (uint32_t)wall_clock64();
-#endif
     {
         const uint32_t* const hs[NR] = {L.s.lh[0], L.s.lh[1], L.s.lh[2]};
         const uint32_t want[NR] = {active[0] ? rank[0] : 0u, active[1] ? rank[1] : 0u, active[2] ? rank[2] : 0u};
@@ -942,9 +927,6 @@ __device__ __forceinline__ void fused_sample(BucketsArg bk, const Geometry& g, c
         if (that < lo) that = lo;
         // every store above must have arrived before the window is published
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#if FUSED_TRACE == 1
-        st[25] = tr_s0; st[27] = tr_s1; st[28] = tr_s2; st[29] = tr_s3; st[30] = tr_s4; st[26] = (uint32_t)wall_clock64();
-#endif
         store16_agent(st + S_LO_KEY, u4a{lo, hi, that, epoch});
     }
     // off the critical path: the histograms of the exact selection, should the select launch need it
@@ -1086,9 +1068,6 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
         }
     }
     const uint32_t lo = L.e.win[0], hi = L.e.win[1], wmul = window_mul(L.e.win[0], L.e.win[1]);
-#if FUSED_TRACE == 1
-    if (threadIdx.x == 0) w.blk_eq[(uint64_t)b * kGroups + grp] = (uint32_t)wall_clock64();
-#endif
     const uint64_t bn = fg.bn;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
@@ -1148,14 +1127,10 @@ __device__ __forceinline__ void fused_bin(BucketsArg bk, const Geometry& g, cons
                     put(cand, cand ? coarse_bin(key, lo, hi, wmul) : 0u, (uint64_t)i | ((uint64_t)v << 32));
                 });
             });
-#if FUSED_TRACE == 1
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (threadIdx.x == 0) w.grp_cnt[((uint64_t)b * kGroups + grp) * kCntStride + 1] = (uint32_t)wall_clock64();
-#endif
 }
 
 // ---- the streaming launch ------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, Workspace w, uint32_t epoch,
+__global__ __launch_bounds__(kBlock, 6) void k_topk_stream(Buckets, Geometry g, Workspace w, uint32_t epoch,
                                                         uint32_t published, uint32_t first_wave,
                                                         uint64_t limit_ticks) {
     const BucketsArg bk = buckets_arg();
@@ -1181,14 +1156,8 @@ __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, 
         b -= 1;
         emit = true;
     }
-#if FUSED_TRACE == 1
-    const uint32_t tr_start = (uint32_t)wall_clock64();
-#endif
     const FusedGeo fg = fused_geo(g, bk, b);
     if (emit) {
-#if FUSED_TRACE == 1
-        if (threadIdx.x == 0 && t < fg.ng) w.blk_above[(uint64_t)b * kGroups + t] = tr_start;
-#endif
         if (t < fg.ng) fused_bin(bk, g, w, b, t, fg, epoch, limit_ticks, L);
         return;
     }
@@ -1226,9 +1195,6 @@ __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, 
     __syncthreads();
     const bool ready = L.a.win[3] != 0;
     const uint32_t lo_key = L.a.win[0], that_key = L.a.win[2];
-#if FUSED_TRACE == 1
-    const uint32_t tr_ready = (uint32_t)wall_clock64();
-#endif
     // both the same in every lane, and kept in scalar registers by saying so at every update
     uint32_t staged = 0;  // candidates of the region so far
     uint32_t dense = 0;   // 1: more candidates than slots
@@ -1353,20 +1319,15 @@ __global__ __launch_bounds__(kBlock, 5) void k_topk_stream(Buckets, Geometry g, 
     // ---- the block counts itself into its group once all its stores have arrived ----------
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-#if FUSED_TRACE == 1
-    if (threadIdx.x == 0) {
-        w.tile_gt[(uint64_t)b * g.tiles + t] = tr_start;
-        w.tile_eq[(uint64_t)b * g.tiles + t] = (uint32_t)wall_clock64();
-        ((uint32_t*)w.blist)[(uint64_t)b * g.tiles + t] = tr_ready;
-    }
-#endif
     if (threadIdx.x == 0)
         __hip_atomic_fetch_add(w.grp_cnt + ((uint64_t)b * kGroups + t / fg.tpg) * kCntStride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The need-th smallest index among the list's entries with key == T: radix select over
-// the index, 11 + 11 + 10 bits.  Called by all threads of the block.
-__device__ __forceinline__ uint32_t resolve_ties64(const uint64_t* l2, uint32_t count2, uint32_t T, uint32_t need,
+// the index, 11 + 11 + 10 bits.  for_list(f) calls f(index, key) for every entry of the list
+// this thread looks at.  Called by all threads of the block.
+template <class ForList>
+__device__ __forceinline__ uint32_t resolve_ties64(ForList&& for_list, uint32_t T, uint32_t need,
                                                    uint32_t* lh /* kBins0 words */, uint32_t* scratch) {
     uint32_t iwant = need, iprefix = 0;
     const int shifts[3] = {21, 10, 0};
@@ -1376,13 +1337,11 @@ __device__ __forceinline__ uint32_t resolve_ties64(const uint64_t* l2, uint32_t 
         for (int i = threadIdx.x; i < kBins0; i += kBlock) lh[i] = 0;
         __syncthreads();
         const int hs = shifts[r] + widths[r];
-        for (uint32_t i = threadIdx.x; i < count2; i += kBlock) {
-            const uint64_t e = l2[i];
-            const uint32_t idx = (uint32_t)e, key = (uint32_t)(e >> 32) & 0x7FFFFFFFu;
+        for_list([&](uint32_t idx, uint32_t key) {
             const bool match = hs >= 32 ? true : ((idx >> hs) == (iprefix >> hs));
             // bins stored reversed, so that pick_bin's top-down scan runs over ascending indices
             if (key == T && match) atomicAdd(&lh[(bins - 1) - ((idx >> shifts[r]) & (bins - 1))], 1u);
-        }
+        });
         __syncthreads();
         uint32_t left;
         const uint32_t rb = pick_bin<kBins0, kBlock>(lh, iwant, 0, &left, scratch);
@@ -1535,13 +1494,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
     const uint32_t b = first_bucket + blockIdx.y, grp = blockIdx.x;
     const FusedGeo fg = fused_geo(g, bk, b);
     if (grp >= fg.ng) return;
-#if FUSED_TRACE == 2
-    uint32_t* tr = w.tile_gt + (uint64_t)b * g.tiles + grp * 8;
-    if (threadIdx.x == 0) tr[0] = (uint32_t)wall_clock64();
-#define TR(i) do { if (threadIdx.x == 0) tr[i] = (uint32_t)wall_clock64(); } while (0)
-#else
-#define TR(i) do {} while (0)
-#endif
     uint32_t* st = w.state + (uint64_t)b * kStateWords;
     uint32_t* out = bucket_wire(g, bk, b);
     // Every load of the first round trip is issued before the first value is looked at, the small
@@ -1567,7 +1519,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
     bool failed = false;
     do {
     // ---- 3: threshold bin from the bucket's counts ------------------------------------------
-    TR(1);
     const uint32_t inc = wave_inclusive_scan(tot[0] + tot[1]);
     const uint64_t reach = __ballot(inc >= k);
     if (!reach) {  // fewer than k candidates
@@ -1616,7 +1567,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
     };
     uint32_t above_before;
     block_exclusive_scan(ab, L.scratch, &above_before);
-    TR(2);
     uint32_t* lh = L.lh;
     const uint32_t bin_lo = window_bin_lo(lo, wmul, jstar);  // smallest key of the threshold bin
     const uint32_t bin_span = window_bin_lo(lo, wmul, jstar + 1) - bin_lo;  // jstar <= kCoarse - 2
@@ -1649,14 +1599,12 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
         want = left;
     }
     if (failed) break;
-    TR(6);
     const uint32_t T = bin_lo + vprefix;
     const uint32_t need2 = want;
     const uint32_t ties = lh[vprefix & (kBinsR - 1)];
     __syncthreads();
     // when only some keys equal to T are taken, they are the need2 lowest indices
-    const uint32_t istar = ties != need2 ? resolve_ties64(l2, n2, T, need2, lh, L.scratch) : 0xFFFFFFFFu;
-    TR(7);
+    const uint32_t istar = ties != need2 ? resolve_ties64(for_list2, T, need2, lh, L.scratch) : 0xFFFFFFFFu;
     auto is_pick = [&](bool valid, uint32_t key, uint32_t idx) {
         return valid && (key > T || (key == T && idx <= istar));
     };
@@ -1676,8 +1624,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
         failed = true;
         break;
     }
-
-    TR(3);
     // ---- 5: payload, in index order -----------------------------------------------------------
     // picks per tile first: the register-held tiles' into rcnt, the others' into the total
     uint32_t w_total = 0;
@@ -1697,7 +1643,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
           });
     if (lane == 0) L.wtot[wave] = w_total;
     __syncthreads();
-    TR(4);
     uint32_t wave_off = above_before + l2_before;
     for (int i = 0; i < wave; i++) wave_off += L.wtot[i];
     auto emit_half = [&](bool valid, uint64_t e, uint32_t pos) {
@@ -1772,7 +1717,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_topk_select(Buckets, Geometry g, 
             return;
         }
     }
-    TR(5);
     if (grp == 0 && threadIdx.x == 0 && !ld_agent(st + S_TIMEOUT)) out[0] = k;
 }
 
@@ -1850,7 +1794,7 @@ bool launch_single_pass(const Buckets& bk, const Geometry& g, const Workspace& w
     // blocks that are resident from the start of the launch: they wait for the sample blocks
     static const int per_cu = [] {
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_topk_stream, kBlock, 0) != hipSuccess || n < 1) n = 5;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_topk_stream, kBlock, 0) != hipSuccess || n < 1) n = 6;
         return n;
     }();
     const uint32_t first_wave = g.nbuckets + (uint32_t)device_info().num_cus * (uint32_t)per_cu;
