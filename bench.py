@@ -148,6 +148,31 @@ def main() -> int:
         extra["stepwise_dropin"] = {"ms": sw["avg_ms"], "GBps": rate((12 * (W - 1) + 8) * N, sw["avg_ms"]),
                                     "bytes_per_elem": 12 * (W - 1) + 8, "launches": nb * (W * (W - 1) + 1)}
 
+        # the same sequence with the folds of one ring step handed over as one list
+        # (mccl_hip_fold2_batch): W - 1 list calls and one scale instead of 855 launches
+        lists = []
+        for j in range(1, W):
+            dl, sl = [], []
+            for b in range(nb):
+                lo, hi = b * BUCKET, min(N, (b + 1) * BUCKET)
+                ce = (hi - lo + W - 1) // W
+                for c in range(W):
+                    s, e = lo + c * ce, min(hi, lo + (c + 1) * ce)
+                    if s < e:
+                        dl.append(out[s:e]); sl.append(ranks[(c + j) % W][s:e])
+            lists.append((dl, sl))
+
+        def step_batched():
+            for dl, sl in lists:
+                ops.fold2_batch(dl, sl, ops.SUM)
+            ops.scale(out, 0.125)
+
+        sb = stats(gpu_time(step_batched, steps=max(3, K // 4), warmup=1)[1])
+        extra["stepwise_batched"] = {"ms": sb["avg_ms"], "GBps": rate((12 * (W - 1) + 8) * N, sb["avg_ms"]),
+                                     "frac": rate((12 * (W - 1) + 8) * N, sb["avg_ms"]) / HBM_PEAK_GBPS,
+                                     "bytes_per_elem": 12 * (W - 1) + 8, "launches": W,
+                                     "note": "host time of building the pointer lists included"}
+
         # ---- config 1: one 25 MiB bucket, W=2, fused (x0 + x1) * 0.5 ------------
         b0, b1 = ranks[0][:BUCKET].clone(), ranks[1][:BUCKET].clone()
         c1 = stats(gpu_time(lambda: ops.fold2_scale(b0, b1, 0.5))[1])

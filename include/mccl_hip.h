@@ -102,6 +102,21 @@ int mccl_hip_pointer_check(const void* ptr, uint64_t nbytes, void** device_ptr);
  * `(src < dst) ? src : dst`.  dst and src need only element alignment. */
 int mccl_hip_fold2(void* dst, const void* src, uint64_t n, int dtype, int op, void* stream);
 
+/* host_dsts[i] = host_dsts[i] (op) host_srcs[i] over host_counts[i] elements, for
+ * i < nfolds: the binary fold above on a list of chunk views, one launch per 128
+ * folds, every fold's result bit-identical to mccl_hip_fold2 on the same pair.
+ * For a caller that holds several folds which do not depend on one another -
+ * the folds of one ring step over all gradient buckets, which the reference
+ * issues one by one (csrc/backend/ProcessGroupMCCL.cpp:492-512, reduce_op ->
+ * metal_accumulate_chunk / cpu_reduce_op per chunk).  The three arrays are host
+ * arrays of device pointers and lengths, read before the call returns.  The
+ * folds run in no particular order: a destination that overlaps any other
+ * fold's destination or source gives MCCL_HIP_ERR_ARG and nothing is launched;
+ * folds of length 0 are skipped. */
+int mccl_hip_fold2_batch(void* const* host_dsts, const void* const* host_srcs,
+                         const uint64_t* host_counts, uint32_t nfolds, int dtype, int op,
+                         void* stream);
+
 /* buf[i] = buf[i] * scale (one fp32 multiply; F16/BF16 multiply in fp32 and
  * round once).  Integral types: T(float(x) * scale), truncating for
  * I64/U8/BOOL and rounding half away from zero for I32.  Replaces

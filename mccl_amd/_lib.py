@@ -22,6 +22,7 @@ SIGNATURES = {
     "mccl_hip_fold2": (_i32, [_vp, _vp, _u64, _i32, _i32, _vp]),
     "mccl_hip_scale": (_i32, [_vp, _u64, _i32, _f32, _vp]),
     "mccl_hip_fold2_scale": (_i32, [_vp, _vp, _u64, _i32, _f32, _vp]),
+    "mccl_hip_fold2_batch": (_i32, [_vp, _vp, _vp, _u32, _i32, _i32, _vp]),
     "mccl_hip_ring_fold": (_i32, [_vp, C.POINTER(_vp), _i32, _u64, _u64, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
     "mccl_hip_topk_k": (_u32, [_u64, _f64]),
     "mccl_hip_topk_max_compressed_size": (_u64, [_u64, _f64]),

@@ -114,6 +114,40 @@ void metal_reduce_op(const at::Tensor& dst, const at::Tensor& src, c10d::ReduceO
     }
 }
 
+void hip_reduce_op_batch(const std::vector<at::Tensor>& dsts, const std::vector<at::Tensor>& srcs,
+                         c10d::ReduceOp::RedOpType op) {
+    std::lock_guard<std::recursive_mutex> lock(g_kernel_mutex);
+    MCCL_CHECK_TENSOR(dsts.size() == srcs.size(), "as many sources as destinations");
+    if (dsts.empty()) return;
+    int code;
+    switch (op) {
+        case c10d::ReduceOp::SUM:
+        case c10d::ReduceOp::AVG: code = MCCL_HIP_SUM; break;
+        case c10d::ReduceOp::MIN: code = MCCL_HIP_MIN; break;
+        case c10d::ReduceOp::MAX: code = MCCL_HIP_MAX; break;
+        case c10d::ReduceOp::PRODUCT: code = MCCL_HIP_PRODUCT; break;
+        default: throw MCCLError("Unsupported ReduceOp: " + std::to_string(static_cast<int>(op)));
+    }
+    std::vector<void*> dp(dsts.size());
+    std::vector<const void*> sp(dsts.size());
+    std::vector<uint64_t> cnt(dsts.size());
+    int device = -1;
+    for (size_t i = 0; i < dsts.size(); i++) {
+        check_same_shape_dtype(dsts[i], srcs[i]);
+        MCCL_CHECK_TENSOR(dsts[i].scalar_type() == dsts[0].scalar_type(), "the pairs of one list share a dtype");
+        HipBufferView d = extract_hip_buffer(dsts[i]);
+        HipBufferView s = extract_hip_buffer(srcs[i]);
+        if (device < 0) device = d.device;
+        MCCL_CHECK_TENSOR(d.device == device && s.device == device, "the pairs of one list live on one device");
+        dp[i] = d.ptr;
+        sp[i] = s.ptr;
+        cnt[i] = static_cast<uint64_t>(safe_numel(dsts[i]));
+    }
+    const int rc = mccl_hip_fold2_batch(dp.data(), sp.data(), cnt.data(), static_cast<uint32_t>(dsts.size()),
+                                        dtype_code(dsts[0], "reduce_op_batch"), code, current_stream(device));
+    throw_on_status(rc, "reduce_op_batch");
+}
+
 uint64_t metal_reduce_op_fenced(const at::Tensor& dst, const at::Tensor& src,
                                 c10d::ReduceOp::RedOpType op) {
     metal_reduce_op(dst, src, op);

@@ -24,6 +24,14 @@ void metal_reduce_op(const at::Tensor& dst, const at::Tensor& src, c10d::ReduceO
 uint64_t metal_reduce_op_fenced(const at::Tensor& dst, const at::Tensor& src,
                                 c10d::ReduceOp::RedOpType op);
 
+/// metal_reduce_op on a list of (dst, src) pairs that do not depend on one another, in one
+/// launch per 128 pairs; every pair's result is bit-identical to metal_reduce_op on it.  No
+/// counterpart in the reference's header: its ring loop issues the folds of one ring step
+/// one by one (csrc/backend/ProcessGroupMCCL.cpp:492-512).  All tensors share dtype and device;
+/// a destination that overlaps another pair's destination or source throws.
+void hip_reduce_op_batch(const std::vector<at::Tensor>& dsts, const std::vector<at::Tensor>& srcs,
+                         c10d::ReduceOp::RedOpType op);
+
 void metal_scale_inplace(const at::Tensor& buf, double scale);
 void metal_accumulate_and_scale(const at::Tensor& dst, const at::Tensor& src, double scale);
 

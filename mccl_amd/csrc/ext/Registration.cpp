@@ -135,6 +135,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         mccl::metal_reduce_op(dst, src, static_cast<c10d::ReduceOp::RedOpType>(op));
         return dst;
     });
+    m.def("_hip_reduce_op_batch", [](const std::vector<at::Tensor>& dsts, const std::vector<at::Tensor>& srcs, int op) {
+        mccl::metal_kernels_init();
+        mccl::hip_reduce_op_batch(dsts, srcs, static_cast<c10d::ReduceOp::RedOpType>(op));
+    }, "dsts[i] (op)= srcs[i] for independent pairs, one launch per 128 pairs");
     m.def("_metal_reduce_op_fenced", [](at::Tensor dst, const at::Tensor& src, int op) {
         mccl::metal_kernels_init();
         return mccl::metal_reduce_op_fenced(dst, src, static_cast<c10d::ReduceOp::RedOpType>(op));

@@ -88,15 +88,16 @@ __device__ __forceinline__ void fold_elem(void* dst, const void* src, uint64_t i
 // ---- binary fold / scale / fused ----------------------------------------------
 // Layout: [head scalars][nvec 16-byte vectors][tail scalars]; head makes the
 // destination 16-byte aligned.
+// block `block` of `nblocks` takes its share of one fold
 template <int DT, int OP, int KIND, bool NT>
-__global__ __launch_bounds__(kBlock) void k_fold2(void* dst, const void* src, uint64_t n,
-                                                  float scale, uint32_t head, uint64_t nvec) {
+__device__ __forceinline__ void fold2_block(void* dst, const void* src, uint64_t n, float scale, uint32_t head,
+                                            uint64_t nvec, uint32_t block, uint32_t nblocks) {
     constexpr int ES = ElemInfo<DT>::size;
     constexpr int EPV = ElemInfo<DT>::per_vec;
     u4a* dv = (u4a*)((char*)dst + (uint64_t)head * ES);
     const char* sv = (const char*)src + (uint64_t)head * ES;
     const uint64_t tile = (uint64_t)kBlock * kUnroll;
-    for (uint64_t base = (uint64_t)blockIdx.x * tile; base < nvec; base += (uint64_t)gridDim.x * tile) {
+    for (uint64_t base = (uint64_t)block * tile; base < nvec; base += (uint64_t)nblocks * tile) {
         u4a d[kUnroll], s[kUnroll];
         if (base + tile <= nvec) {
 #pragma unroll
@@ -131,26 +132,69 @@ __global__ __launch_bounds__(kBlock) void k_fold2(void* dst, const void* src, ui
         }
     }
     // scalar head and tail (fewer than EPV elements each)
-    const uint64_t g = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t g = (uint64_t)block * kBlock + threadIdx.x;
     if (g < head) fold_elem<DT, OP, KIND>(dst, src, g, scale);
     const uint64_t tail = head + nvec * EPV;
     if (g < (uint64_t)EPV && tail + g < n) fold_elem<DT, OP, KIND>(dst, src, tail + g, scale);
+}
+
+template <int DT, int OP, int KIND, bool NT>
+__global__ __launch_bounds__(kBlock) void k_fold2(void* dst, const void* src, uint64_t n,
+                                                  float scale, uint32_t head, uint64_t nvec) {
+    fold2_block<DT, OP, KIND, NT>(dst, src, n, scale, head, nvec, blockIdx.x, gridDim.x);
+}
+
+// ---- a list of independent binary folds in one launch ---------------------------
+// blockIdx.y = fold, blockIdx.x strides over that fold's vectors.  The table is read where
+// the launch put it, in the kernel-argument segment, through scalar loads (indexing the
+// by-value parameter would make the compiler copy it to per-lane scratch memory first): it
+// is therefore the only parameter.
+constexpr int kFoldBatch = 128;  // folds per launch
+struct FoldBatch {
+    void* dst[kFoldBatch];
+    const void* src[kFoldBatch];
+    uint64_t n[kFoldBatch];
+};
+template <int DT, int OP, bool NT>
+__global__ __launch_bounds__(kBlock) void k_fold2_batch(FoldBatch) {
+    typedef const __attribute__((address_space(4))) FoldBatch* Arg;
+    const Arg fb = (Arg)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr int ES = ElemInfo<DT>::size;
+    constexpr int EPV = ElemInfo<DT>::per_vec;
+    void* dst = fb->dst[blockIdx.y];
+    const void* src = fb->src[blockIdx.y];
+    const uint64_t n = fb->n[blockIdx.y];
+    uint64_t head = ((16 - ((uintptr_t)dst & 15)) & 15) / ES;
+    if (head > n) head = n;
+    const uint64_t nvec = (n - head) / EPV;
+    fold2_block<DT, OP, 0, NT>(dst, src, n, 1.0f, (uint32_t)head, nvec, blockIdx.x, gridDim.x);
 }
 
 // ---- integral types (DDP metadata, counters): plain grid-stride ---------------
 // Wrap-around arithmetic, bool folded as raw uint8
 // (csrc/metal/AccelerateOps.mm:206-236, csrc/metal/shaders.metal:554-731).
 template <typename T, int OP>
-__global__ __launch_bounds__(kBlock) void k_fold2_int(T* dst, const T* src, uint64_t n) {
+__device__ __forceinline__ T fold_int(T d, T s) {
     typedef typename std::make_unsigned<T>::type UT;
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) {
-        T d = dst[i], s = src[i];
-        if constexpr (OP == kAdd) d = (T)((UT)d + (UT)s);
-        else if constexpr (OP == kMul) d = (T)((UT)d * (UT)s);
-        else if constexpr (OP == kMin) d = s < d ? s : d;
-        else d = s > d ? s : d;
-        dst[i] = d;
-    }
+    if constexpr (OP == kAdd) return (T)((UT)d + (UT)s);
+    else if constexpr (OP == kMul) return (T)((UT)d * (UT)s);
+    else if constexpr (OP == kMin) return s < d ? s : d;
+    else return s > d ? s : d;
+}
+template <typename T, int OP>
+__global__ __launch_bounds__(kBlock) void k_fold2_int(T* dst, const T* src, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock)
+        dst[i] = fold_int<T, OP>(dst[i], src[i]);
+}
+template <typename T, int OP>
+__global__ __launch_bounds__(kBlock) void k_fold2_batch_int(FoldBatch) {
+    typedef const __attribute__((address_space(4))) FoldBatch* Arg;
+    const Arg fb = (Arg)__builtin_amdgcn_kernarg_segment_ptr();
+    T* dst = (T*)fb->dst[blockIdx.y];
+    const T* src = (const T*)fb->src[blockIdx.y];
+    const uint64_t n = fb->n[blockIdx.y];
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock)
+        dst[i] = fold_int<T, OP>(dst[i], src[i]);
 }
 
 // T(float(x) * scale): int32 rounds half away from zero, int64 / uint8 truncate
@@ -385,6 +429,68 @@ int launch_fold2_int(void* dst, const void* src, uint64_t n, int opi, hipStream_
     return launch_status();
 }
 
+// One launch per kFoldBatch folds.  x covers the longest fold of the launch (shorter folds' surplus
+// blocks leave at once), capped so that the whole grid stays within the streaming kernels' bound.
+template <class Launch>
+int launch_batches(void* const* dsts, const void* const* srcs, const uint64_t* counts, uint32_t nfolds,
+                   uint64_t elems_per_block, Launch&& launch) {
+    const uint64_t cap = (uint64_t)device_info().num_cus * (uint64_t)tuning().fold_blocks_per_cu;
+    FoldBatch fb;
+    uint32_t m = 0;
+    uint64_t longest = 0;
+    auto flush = [&]() {
+        if (m == 0) return;
+        for (uint32_t i = m; i < (uint32_t)kFoldBatch; i++) { fb.dst[i] = nullptr; fb.src[i] = nullptr; fb.n[i] = 0; }
+        const uint64_t want = (longest + elems_per_block - 1) / elems_per_block;
+        launch(fb, dim3(clamp_u32(want, 1, cap / m > 0 ? cap / m : 1), m, 1));
+        m = 0;
+        longest = 0;
+    };
+    for (uint32_t i = 0; i < nfolds; i++) {
+        if (counts[i] == 0) continue;
+        fb.dst[m] = dsts[i];
+        fb.src[m] = srcs[i];
+        fb.n[m] = counts[i];
+        longest = counts[i] > longest ? counts[i] : longest;
+        if (++m == (uint32_t)kFoldBatch) flush();
+    }
+    flush();
+    return launch_status();
+}
+
+template <int DT, int OP>
+int launch_fold2_batch_t(void* const* dsts, const void* const* srcs, const uint64_t* counts, uint32_t nfolds,
+                         hipStream_t st) {
+    const uint64_t per_block = (uint64_t)kBlock * kUnroll * ElemInfo<DT>::per_vec;
+    const bool nt = tuning().nontemporal != 0;
+    return launch_batches(dsts, srcs, counts, nfolds, per_block, [&](const FoldBatch& fb, dim3 grid) {
+        if (nt) k_fold2_batch<DT, OP, true><<<grid, kBlock, 0, st>>>(fb);
+        else k_fold2_batch<DT, OP, false><<<grid, kBlock, 0, st>>>(fb);
+    });
+}
+template <int DT>
+int launch_fold2_batch_dt(void* const* dsts, const void* const* srcs, const uint64_t* counts, uint32_t nfolds,
+                          int opi, hipStream_t st) {
+    switch (opi) {
+        case kAdd: return launch_fold2_batch_t<DT, kAdd>(dsts, srcs, counts, nfolds, st);
+        case kMul: return launch_fold2_batch_t<DT, kMul>(dsts, srcs, counts, nfolds, st);
+        case kMin: return launch_fold2_batch_t<DT, kMin>(dsts, srcs, counts, nfolds, st);
+        default: return launch_fold2_batch_t<DT, kMax>(dsts, srcs, counts, nfolds, st);
+    }
+}
+template <typename T>
+int launch_fold2_batch_int(void* const* dsts, const void* const* srcs, const uint64_t* counts, uint32_t nfolds,
+                           int opi, hipStream_t st) {
+    return launch_batches(dsts, srcs, counts, nfolds, kBlock, [&](const FoldBatch& fb, dim3 grid) {
+        switch (opi) {
+            case kAdd: k_fold2_batch_int<T, kAdd><<<grid, kBlock, 0, st>>>(fb); break;
+            case kMul: k_fold2_batch_int<T, kMul><<<grid, kBlock, 0, st>>>(fb); break;
+            case kMin: k_fold2_batch_int<T, kMin><<<grid, kBlock, 0, st>>>(fb); break;
+            default: k_fold2_batch_int<T, kMax><<<grid, kBlock, 0, st>>>(fb); break;
+        }
+    });
+}
+
 template <typename T>
 int launch_scale_int(void* buf, uint64_t n, float scale, hipStream_t st) {
     const uint32_t blocks = stream_blocks((n + kBlock - 1) / kBlock);
@@ -472,6 +578,49 @@ int mccl_hip_fold2(void* dst, const void* src, uint64_t n, int dtype, int op, vo
         case MCCL_HIP_BOOL:
         case MCCL_HIP_U8: return launch_fold2_int<uint8_t>(dst, src, n, opi, st);
         default: return MCCL_HIP_ERR_DTYPE;
+    }
+}
+
+int mccl_hip_fold2_batch(void* const* host_dsts, const void* const* host_srcs, const uint64_t* host_counts,
+                         uint32_t nfolds, int dtype, int op, void* stream) {
+    const int opi = op_index(op);
+    if (opi < 0) return MCCL_HIP_ERR_OP;
+    if (nfolds == 0) return MCCL_HIP_OK;
+    if (!host_dsts || !host_srcs || !host_counts) return MCCL_HIP_ERR_ARG;
+    int es;
+    switch (dtype) {
+        case MCCL_HIP_F32: case MCCL_HIP_I32: es = 4; break;
+        case MCCL_HIP_F16: case MCCL_HIP_BF16: es = 2; break;
+        case MCCL_HIP_I64: es = 8; break;
+        case MCCL_HIP_BOOL: case MCCL_HIP_U8: es = 1; break;
+        default: return MCCL_HIP_ERR_DTYPE;
+    }
+    for (uint32_t i = 0; i < nfolds; i++) {
+        if (host_counts[i] == 0) continue;
+        if (!host_dsts[i] || !host_srcs[i] || host_counts[i] > MCCL_HIP_MAX_ELEMS) return MCCL_HIP_ERR_ARG;
+    }
+    // the folds of one call run in no particular order: a destination may not overlap any other
+    // fold's destination or source
+    for (uint32_t i = 0; i < nfolds; i++) {
+        if (host_counts[i] == 0) continue;
+        const uintptr_t d0 = (uintptr_t)host_dsts[i], d1 = d0 + host_counts[i] * (uint64_t)es;
+        for (uint32_t j = 0; j < nfolds; j++) {
+            if (j == i || host_counts[j] == 0) continue;
+            const uint64_t bytes = host_counts[j] * (uint64_t)es;
+            const uintptr_t a0 = (uintptr_t)host_dsts[j], b0 = (uintptr_t)host_srcs[j];
+            if ((d0 < a0 + bytes && a0 < d1) || (d0 < b0 + bytes && b0 < d1)) return MCCL_HIP_ERR_ARG;
+        }
+    }
+    int rc = mccl_hip_init();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case MCCL_HIP_F32: return launch_fold2_batch_dt<MCCL_HIP_F32>(host_dsts, host_srcs, host_counts, nfolds, opi, st);
+        case MCCL_HIP_F16: return launch_fold2_batch_dt<MCCL_HIP_F16>(host_dsts, host_srcs, host_counts, nfolds, opi, st);
+        case MCCL_HIP_BF16: return launch_fold2_batch_dt<MCCL_HIP_BF16>(host_dsts, host_srcs, host_counts, nfolds, opi, st);
+        case MCCL_HIP_I32: return launch_fold2_batch_int<int32_t>(host_dsts, host_srcs, host_counts, nfolds, opi, st);
+        case MCCL_HIP_I64: return launch_fold2_batch_int<int64_t>(host_dsts, host_srcs, host_counts, nfolds, opi, st);
+        default: return launch_fold2_batch_int<uint8_t>(host_dsts, host_srcs, host_counts, nfolds, opi, st);
     }
 }
 

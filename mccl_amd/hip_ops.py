@@ -59,6 +59,23 @@ def fold2(dst: torch.Tensor, src: torch.Tensor, op: int = SUM) -> torch.Tensor:
     return dst
 
 
+def fold2_batch(dsts: Sequence[torch.Tensor], srcs: Sequence[torch.Tensor], op: int = SUM) -> None:
+    """dsts[i] (op)= srcs[i] for every i, in one launch per 128 folds.  The folds run in no
+    particular order: a destination may not overlap any other fold's destination or source
+    (the library refuses such a list)."""
+    if len(dsts) != len(srcs):
+        raise ValueError("as many sources as destinations")
+    if not dsts:
+        return
+    for d, s_ in zip(dsts, srcs):
+        _dev(d, "dst"); _dev(s_, "src")
+        if d.shape != s_.shape or d.dtype != s_.dtype or d.dtype != dsts[0].dtype:
+            raise ValueError("shape / dtype mismatch")
+    counts = (C.c_uint64 * len(dsts))(*[d.numel() for d in dsts])
+    rc = _lib.load().mccl_hip_fold2_batch(_ptrs(dsts), _ptrs(srcs), counts, len(dsts), dtype_code(dsts[0]), op, _stream())
+    _lib.check(rc, "fold2_batch")
+
+
 def scale(buf: torch.Tensor, s: float) -> torch.Tensor:
     _dev(buf, "buf")
     rc = _lib.load().mccl_hip_scale(buf.data_ptr(), buf.numel(), dtype_code(buf), s, _stream())

@@ -114,6 +114,32 @@ class TestScaleAndFused:
         assert torch.equal(k["acc_scale"](t([1., 3., 5.], h), t([3., 5., 7.], h), 0.5), t([2., 4., 6.], h))
 
 
+def test_reduce_op_batch_equals_reduce_op_pair_by_pair(k):
+    C = k["C"]
+    g = torch.Generator(device=DEV).manual_seed(5)
+    sizes = [1, 7, 4096, 100_003, 5]
+    for dt in (torch.float32, torch.bfloat16, torch.int64):
+        def mk():
+            if dt == torch.int64:
+                return [torch.randint(-10**9, 10**9, (n,), generator=g, device=DEV) for n in sizes]
+            return [torch.randn(n, generator=g, device=DEV).to(dt) for n in sizes]
+        d0, s0 = mk(), mk()
+        for op in (0, 3, 4):  # SUM, MIN, MAX
+            one = [x.clone() for x in d0]
+            many = [x.clone() for x in d0]
+            for d, s_ in zip(one, s0):
+                C._metal_reduce_op(d, s_, op)
+            C._hip_reduce_op_batch(many, s0, op)
+            for a, b in zip(one, many):
+                assert torch.equal(a, b)
+    x = torch.zeros(100, device=DEV)
+    with pytest.raises(RuntimeError):
+        C._hip_reduce_op_batch([x[:60], x[50:]], [torch.ones(60, device=DEV), torch.ones(50, device=DEV)], 0)
+    with pytest.raises(RuntimeError, match="Dtype mismatch"):
+        C._hip_reduce_op_batch([x], [torch.ones(100, device=DEV, dtype=torch.float16)], 0)
+    C._hip_reduce_op_batch([], [], 0)
+
+
 def test_errors_and_fenced_reduce(k):
     C = k["C"]
     with pytest.raises(RuntimeError, match="Shape mismatch"):

@@ -73,6 +73,51 @@ def test_ring_fold_equals_stepwise_binary_folds_on_chunk_views(ops):
     assert torch.equal(out.view(torch.int32), step.view(torch.int32))
 
 
+@pytest.mark.parametrize("dt,op", [(F32, OP_SUM), (oracle.BF16, OP_SUM), (oracle.F16, oracle.OP_MAX), (oracle.I32, OP_SUM)])
+def test_batched_folds_equal_the_per_call_sequence(ops, dt, op):
+    # the same step-wise sequence with the folds of one ring step handed over as one list: ws rank
+    # buffers, 3 buckets (the last one shorter and odd), every bucket in ws chunks; ring step j
+    # folds chunk (r - j) of rank r - 1's partial into rank r's copy, for all r and buckets at once
+    ws, n, be = 4, 700_003, 262_144
+    rng = np.random.default_rng(17)
+    if dt == oracle.I32:
+        ins = [rng.integers(-2**31, 2**31, n, dtype=np.int64).astype(np.int32) for _ in range(ws)]
+    else:
+        ins = [rand_vals(rng, n, dt, sigma=1e-3, specials=False) for _ in range(ws)]
+    one = [to_dev(x, dt, pad_front=r % 3) for r, x in enumerate(ins)]     # folded call by call
+    many = [to_dev(x, dt, pad_front=r % 3) for r, x in enumerate(ins)]    # folded list by list
+    for j in range(1, ws):
+        dsts, srcs, d1, s1 = [], [], [], []
+        for lo in range(0, n, be):
+            hi = min(n, lo + be)
+            ce = (hi - lo + ws - 1) // ws
+            for r in range(ws):
+                c = (r - j) % ws
+                a, b = lo + c * ce, min(hi, lo + (c + 1) * ce)
+                if a >= b:
+                    continue
+                dsts.append(many[r][a:b]); srcs.append(many[(r - 1) % ws][a:b])
+                d1.append(one[r][a:b]); s1.append(one[(r - 1) % ws][a:b])
+        ops.fold2_batch(dsts, srcs, op)
+        for d, s_ in zip(d1, s1):
+            ops.fold2(d, s_, op)
+    for a, b in zip(one, many):
+        assert np.array_equal(bits(to_np(a, dt)), bits(to_np(b, dt)))
+
+
+def test_batched_folds_refuse_overlapping_destinations(ops):
+    x = torch.zeros(1000, device=DEV)
+    y = torch.ones(1000, device=DEV)
+    with pytest.raises(Exception):
+        ops.fold2_batch([x[:600], x[500:]], [y[:600], y[500:]], OP_SUM)      # two destinations overlap
+    with pytest.raises(Exception):
+        ops.fold2_batch([x[:500], y[:500]], [y[:500], x[500:]], OP_SUM)      # a destination is another fold's source
+    assert float(x.sum()) == 0.0 and float(y.sum()) == 1000.0                  # nothing was launched
+    ops.fold2_batch([], [], OP_SUM)
+    ops.fold2_batch([x[:0], x[:500]], [y[:0], y[:500]], OP_SUM)               # empty folds are skipped
+    assert float(x.sum()) == 500.0
+
+
 @pytest.mark.parametrize("dt", [F16, BF16])
 @pytest.mark.parametrize("stepwise", [False, True])
 def test_half_ring_fold_matches_oracle(ops, dt, stepwise):
