@@ -1,6 +1,7 @@
 // Backend options exposed to Python; field names and defaults follow
-// csrc/backend/Options.hpp:12-45.  Only compression, topk_ratio, fast_math and
-// gpu_threshold mean something to this build (no transport, no engine).
+// csrc/backend/Options.hpp:12-45.  Only compression and topk_ratio change what this
+// build does (no transport, no engine); fast_math and gpu_threshold are accepted and
+// ignored: there is one arithmetic (IEEE, no contraction) and no host fold to fall back to.
 #pragma once
 
 #include <torch/csrc/distributed/c10d/Backend.hpp>

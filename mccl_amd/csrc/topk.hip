@@ -570,7 +570,7 @@ __device__ __forceinline__ bool bucket_barrier(uint32_t* counter, uint32_t parti
 //                   tiles (at most 64 groups per bucket).
 //   bin blocks      64 per bucket.  Block g waits until group g's tiles are finished (when it
 //                   is dispatched - one bucket later - they are, except in the last bucket),
-//                   counts the group's candidates per coarse window bin (64 bins), publishes
+//                   counts the group's candidates per coarse window bin (128 bins), publishes
 //                   the counts and copies the candidates, binned, to the bucket's per-bin
 //                   lists.  It waits for nothing else.
 // k_topk_select - 64 blocks per bucket; nothing crosses blocks any more: every block
@@ -593,7 +593,17 @@ __device__ __forceinline__ bool bucket_barrier(uint32_t* counter, uint32_t parti
 // emitter, the slowest XCD collects every emitter, slows down further and jams; with
 // dedicated selection blocks in the grid nothing jams, but every dependent memory round trip
 // of the selection takes 5 to 8 microseconds while the stream is in flight, the blocks live
-// 50 to 100 microseconds each, and the stream loses a quarter of its block slots to them.)
+// 50 to 100 microseconds each, and the stream loses a quarter of its block slots to them.
+// With every bucket's selection blocks at the very end of the grid the launch boundary
+// disappears, but the kernel then carries the selection's registers: at 125 registers four
+// blocks fit a CU instead of six and the stream - whose blocks idle while their stores are
+// acknowledged - takes 15.3 microseconds per bucket instead of 11.8; trimmed to 89 registers
+// it streams at 12.6, while the bin blocks' lists and counts have to be written through
+// (scattered 8-byte stores, a memory transaction each: 10 microseconds per call; an L2
+// write-back per bin block instead costs 380) and every selection block reads its bucket's
+// list past its L2.  Whole call 228 microseconds against 221 for the two launches.  Two tiles
+// per streaming block, the second tile's loads under way while the first tile's stores are
+// acknowledged, stream slower as well: 220 against 205 microseconds.)
 // All waits are bounded all the same (`limit_ticks`): a block that gives up sets S_TIMEOUT,
 // overwrites the bucket's payload header with kPoisonK and leaves; k_topk_select leaves such
 // a bucket alone.

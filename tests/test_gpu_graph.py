@@ -1,6 +1,7 @@
 """The entry points only enqueue kernels on the caller's stream (no host
 synchronisation, no allocation, no memset nodes), so a launch-bound sequence
-such as the six launches of a one-bucket top-k compress can be captured in a HIP
+such as the launches of a one-bucket top-k compress (two on the single-pass path, six on the
+exact path) can be captured in a HIP
 graph.  Every replay is checked against the eager result and the oracle, with
 eager work and synchronisations in between."""
 import numpy as np
