@@ -353,7 +353,8 @@ def main() -> int:
                         part = local
                     oracle.scale(part, oracle.F32, 0.125, threads=0)
             times.append(time.perf_counter() - t0)
-            if time.perf_counter() - t_all > 10.0 or len(times) >= 12:
+            spent = time.perf_counter() - t_all
+            if spent > 10.0 or (len(times) >= 12 and spent > 3.0):   # at least 3 s of folding, at most 10
                 break
         reps = len(times)
         cpu_s = sum(times) / reps
